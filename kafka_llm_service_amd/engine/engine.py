@@ -71,6 +71,9 @@ class EngineConfig:
     # the group (step_lockstep; planned ahead like step())
     dp_attention: bool = False
     eos_token_ids: list[int] = field(default_factory=list)
+    # activation / weight dtype: "bfloat16", or "float32" (every matrix product and activation in true fp32) for the
+    # model families whose kernels are built for it (Budurax)
+    dtype: str = "bfloat16"
 
     def resolve_device(self) -> torch.device:
         if self.device:
@@ -127,10 +130,19 @@ class LLMEngine:
 
             st = pstate.get()
             dpa = (st.ep, st.ep_rank)
+        if cfg.dtype not in ("bfloat16", "float32"):
+            raise ValueError(f"dtype {cfg.dtype!r}: bfloat16 or float32")
+        if cfg.dtype == "float32":
+            torch.backends.cuda.matmul.allow_tf32 = False  # true fp32 products (no reduced-precision matrix mode)
+            torch.set_float32_matmul_precision("highest")
         self.model = model or build_model(mc, self.device, tp=cfg.tp, tp_rank=cfg.tp_rank, seed=cfg.seed,
                                           weights=cfg.weights, max_positions=min(cfg.max_model_len,
                                                                                  mc.max_position_embeddings),
-                                          dp_attention=dpa)
+                                          dp_attention=dpa, dtype=getattr(torch, cfg.dtype))
+        self.slots = None
+        if getattr(self.model, "plan", "") == "segments":
+            self._init_segments(cfg, mc, t0)
+            return
         mode = os.environ.get("KAFKA_DECODE_GEMM", cfg.decode_gemm)
         if mode == "auto":
             mode = "stream" if self.device.type == "cuda" else "blas"
@@ -211,6 +223,103 @@ class LLMEngine:
         self.stop_checker_factory = None  # set by the frontend: (request params) -> incremental stop-string checker
         log.info("engine ready: %s tp=%d kv pages=%d (%s, %.1f GB) load %.1fs", mc.name, cfg.tp, nb, cfg.kv_dtype,
                  nb * page_bytes / 1e9, self.load_s)
+
+    def _init_segments(self, cfg: EngineConfig, mc, t0: float) -> None:
+        """Caches and scheduler of a segment-planned model (models/budurax.py): latent page pools sized like the KV
+        pool, one recurrent-state slot per live sequence. Recurrent state cannot be shared through the prefix tree
+        (a cached page says nothing about the state behind it), so the prefix cache is off and every prompt is
+        computed from its first token."""
+        from kafka_llm_service_amd.runtime import StateSlots
+
+        self.load_s = time.perf_counter() - t0
+        self.eos = set(cfg.eos_token_ids or mc.eos_token_ids)
+        self.fi = faults.get()
+        page_bytes = self.model.page_bytes()
+        if self.fi.kv_blocks:
+            nb = self.fi.kv_blocks
+        elif cfg.num_kv_blocks:
+            nb = cfg.num_kv_blocks
+        elif self.device.type == "cuda":
+            free, _ = torch.cuda.mem_get_info(self.device)
+            nb = int(free * cfg.kv_fraction) // page_bytes
+        else:
+            nb = 4096
+        self.num_blocks = nb
+        pages, state = self.model.alloc_cache(nb, cfg.max_num_seqs)
+        self.k_cache, self.v_cache = pages, state
+        self.kvm = KVManager(nb, 16, False, cfg.kv_run_pages)
+        self.slots = StateSlots(cfg.max_num_seqs)
+        max_blocks = (cfg.max_model_len + 15) // 16
+        self.sched = Scheduler(SchedulerConfig(max_num_seqs=cfg.max_num_seqs,
+                                               max_num_batched_tokens=cfg.max_num_batched_tokens,
+                                               max_prefill_chunk=cfg.max_prefill_chunk,
+                                               prefill_tokens_while_decoding=cfg.prefill_tokens_while_decoding,
+                                               prefill_cost_budget=0, max_model_len=cfg.max_model_len,
+                                               max_blocks_per_seq=max_blocks), self.kvm, slots=self.slots)
+        self.runner = ModelRunner(self.model, pages, state, self.kvm, cfg.max_num_seqs, max_blocks, slots=self.slots)
+        cfg.use_graphs = False
+        self.requests = {}
+        self.stats = {"steps": 0, "prompt_tokens": 0, "cached_tokens": 0, "output_tokens": 0, "step_time": 0.0,
+                      "replans": 0, "planned_ahead": 0, "planned_late": 0}
+        self.host_s = {"plan": 0.0, "launch": 0.0, "wait": 0.0, "finish": 0.0}
+        self._inflight = None
+        self.step_ms = deque(maxlen=512)
+        self._t_done = 0.0
+        self._coll_mark = (0, 0)
+        self._n_added = 0
+        self.stop_checker_factory = None
+        log.info("engine ready: %s (%s) latent pages=%d (%.2f GB) state slots=%d (%.2f GB) load %.1fs", mc.name,
+                 cfg.dtype, nb, nb * page_bytes / 1e9, cfg.max_num_seqs, state.nbytes() / 1e9, self.load_s)
+
+    # trace replay -----------------------------------------------------------------------------------------------
+    @torch.inference_mode()
+    def feed(self, entries: list[tuple[str, list[int], list[int]]], end: list[str] = (),
+             layers_out: list | None = None) -> torch.Tensor:
+        """Run exactly the given next tokens of the given requests as ONE step and return fp32 logits [rows, V] for
+        the wanted places — (request id, tokens, offsets among these tokens) per entry, rows in the order of the
+        entries and of their offsets. A request is admitted at its first entry; ``end`` lists the requests whose
+        pages and state slot are given back after the step. Nothing is sampled. The step goes through the engine's
+        scheduler bookkeeping, page and slot managers, plan builder and model step like a generated one."""
+        if self._inflight is not None:
+            raise RuntimeError("feed() while a generation step is in flight")
+        portions, want = [], {}
+        for rid, toks, offs in entries:
+            toks = [int(t) for t in toks]
+            V = self.model_cfg.vocab_size
+            if not toks or min(toks) < 0 or max(toks) >= V:
+                raise ValueError(f"request {rid}: token ids must lie in [0, {V}) and a portion cannot be empty")
+            seq = self.requests.get(rid)
+            if seq is None:
+                seq = Sequence(rid, toks, SamplingParams(max_tokens=1))
+                self.requests[rid] = seq
+            else:
+                if seq.num_computed != seq.total_len:
+                    raise RuntimeError(f"request {rid} has uncomputed tokens")
+                seq.prompt_ids.extend(toks)
+                self.kvm.append_tokens(seq.seq_id, toks)
+            portions.append((seq, len(toks)))
+            want[seq.seq_id] = [int(o) for o in offs]
+        logits = None
+        if portions:
+            batch = self.sched.replay(portions)
+            host, _ = self.runner.build_host(batch, want=want)
+            logits = self.runner.forward_logits(host, layers_out=layers_out)
+            for s, n in portions:
+                s.num_computed += n
+                self.kvm.commit(s.seq_id, s.num_computed)
+            self.stats["steps"] += 1
+            # rows come back in plan order (single tokens first); hand them out in the caller's order
+            at = {k: i for i, k in enumerate(host.owners)}
+            order = [at[(s.seq_id, o)] for s, _ in portions for o in want[s.seq_id]]
+            if order != list(range(len(order))):
+                logits = logits.index_select(0, torch.tensor(order, dtype=torch.long, device=logits.device))
+        for rid in end:
+            seq = self.requests.pop(rid, None)
+            if seq is not None:
+                self.sched.finish(seq, "stop")
+        if logits is None:
+            logits = torch.empty(0, self.model_cfg.vocab_size)
+        return logits.float()
 
     # ------------------------------------------------------------------------------------------------------------
 

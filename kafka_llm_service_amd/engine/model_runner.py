@@ -57,6 +57,10 @@ class HostStep:
     # i64[late_off + n_late : +n_late] = source rows of the previous step's sampler output
     n_late: int = 0
     late_off: int = 0
+    # segment plans (models whose ``plan`` is "segments": one run of rows per sequence): i32 = block tables [n_seg,
+    # bt_w] | row -> run [T] | runs [n_seg, 4] = (first row, rows, first position, state slot)
+    n_seg: int = 0
+    owners: list = field(default_factory=list)  # with ``want``: (seq_id, offset) of every logit row, in row order
 
 
 @dataclass
@@ -73,7 +77,7 @@ class SampleParams:
 
 
 _PLAN_SCALARS = ("B", "T", "nbt", "bt_w", "n_rows", "s_total", "n_dec_items", "n_prefix_items", "cascade_prefix",
-                 "n_items", "prefill_splits", "n_merge", "n_late", "late_off", "bt_need", "prefix_joined")
+                 "n_items", "prefill_splits", "n_merge", "n_late", "late_off", "bt_need", "prefix_joined", "n_seg")
 PLAN_HDR = 32  # int64 header of a broadcast step plan
 PLAN_PAYLOAD_IDX = 1 + len(_PLAN_SCALARS) + 4  # header word holding the payload size (pack_plan)
 
@@ -470,13 +474,20 @@ class _Stager:
 class ModelRunner:
     def __init__(self, model: TransformerLM, k_caches, v_caches, kvm, max_num_seqs: int, max_blocks_per_seq: int,
                  cascade_min_prefix: int = 512, use_cascade: bool = True, target_wgs: int = 256,
-                 prefill_kv_chunk: int = 1024):
+                 prefill_kv_chunk: int = 1024, slots=None):
         self.model = model
+        # paged K / V pools per layer — or, for a model planned as segments, its per-layer page pools and its
+        # per-slot recurrent state (models/budurax.py alloc_cache)
         self.k_caches, self.v_caches = k_caches, v_caches
         self.kvm = kvm
+        self.slots = slots  # runtime.StateSlots of a model with per-sequence recurrent state
         self.device = model.device
         self.max_num_seqs = max_num_seqs
         self.max_blocks = max_blocks_per_seq
+        self.segments = getattr(model, "plan", "") == "segments"
+        if self.segments:
+            self._init_common(max_num_seqs)
+            return
         self.G = model.hq // model.hkv
         # tile-kernel variant (ops.tile_rows): 3 = LDS-DMA ring kernel (csrc/attn_tile.hip, 8 waves x 256 query rows,
         # bf16 pages); 0 = register-staged 8 waves x 256 rows (fp8 pages); 1 = 4 waves x 128 rows
@@ -520,18 +531,86 @@ class ModelRunner:
         # grammar masks / forced tokens / penalties inside the sampler kernel (tables allocated on first use)
         self.lp = LogitsProcessor(self.device, self.vocab, max_slots=max(256, max_num_seqs))
 
+    def _init_common(self, max_num_seqs: int) -> None:
+        """The runner state every plan kind needs (a segment-planned model has no tile variants or cascade)."""
+        self.variant, self.pad_rows, self.use_cascade, self.graphs = 0, False, False, None
+        self.vocab = self.model.cfg.vocab_size
+        self._pin = self.device.type == "cuda"
+        self.last_stats = {}
+        self.recent_stats = deque(maxlen=16)
+        self.rows_hist = [0] * len(ROWS_BUCKETS)
+        self.broadcast = None
+        self._tok_host = None
+        self._err_host = None
+        self.stager = _Stager(self.device)
+        self.tok_buf = torch.zeros(max_num_seqs * 2 + 64, dtype=torch.int64, device=self.device)
+        self.step_events = None
+        self.lp = LogitsProcessor(self.device, self.vocab, max_slots=max(256, max_num_seqs))
+
     # ------------------------------------------------------------------------------------------------------------
     def prepare(self, batch: ScheduledBatch) -> tuple[StepInput, list[Sequence]]:
         host, sample_seqs = self.build_host(batch)
         return self.to_device(host), sample_seqs
 
-    def build_host(self, batch: ScheduledBatch) -> tuple[HostStep, list[Sequence]]:
-        """All host-side work of a step: token/slot/page-table packing and attention work-item planning. The result
+    def _build_host_segments(self, batch: ScheduledBatch, want: dict | None) -> tuple[HostStep, list[Sequence]]:
+        """The plan of a segment-planned model: every sequence of the step is one run of consecutive rows (a decode
+        row is a run of one) with its first position, its state slot and its page list; the kernels need no other
+        work items. Same int64 pack as the paged-attention plan (tokens | positions | slots | logit rows), so pending
+        decode inputs are patched the same way."""
+        runs = [(s, s.total_len - 1, s.total_len) for s in batch.decode] + list(batch.prefill)
+        R = len(runs)
+        T = sum(b - a for _, a, b in runs)
+        need = max([-(-b // PAGE) for _, _, b in runs] + [1])
+        bt_w = min(self.max_blocks, -(-need // 16) * 16)
+        bt = np.zeros((max(1, R), bt_w), dtype=np.int32)
+        if R:
+            self.kvm.fill_block_tables([s.seq_id for s, _, _ in runs], bt)
+        tokens = np.empty(T, dtype=np.int64)
+        positions = np.empty(T, dtype=np.int64)
+        slots = np.empty(T, dtype=np.int64)
+        tok_seg = np.empty(T, dtype=np.int32)
+        seg = np.zeros((max(1, R), 4), dtype=np.int32)
+        sample_seqs, logit_rows, patch, owners = [], [], [], []
+        r = 0
+        for j, (s, a, b) in enumerate(runs):
+            n = b - a
+            toks = s.tokens_range(a, b)
+            tokens[r:r + n] = toks
+            if n == 1 and toks[0] < 0:  # PENDING: sampled by the step still in flight
+                patch.append((r, s, a))
+            positions[r:r + n] = np.arange(a, b)
+            self.kvm.fill_slots(s.seq_id, a, b, slots, r)
+            tok_seg[r:r + n] = j
+            seg[j] = (r, n, a, self.slots.slot_of(s.seq_id) if self.slots is not None else 0)
+            if want is not None:
+                offs = want.get(s.seq_id, ())
+                if any(o < 0 or o >= n for o in offs):
+                    raise ValueError("a wanted row lies outside the sequence's portion of this step")
+                logit_rows += [r + o for o in offs]
+                owners += [(s.seq_id, o) for o in offs]
+            elif b == s.total_len:
+                sample_seqs.append(s)
+                logit_rows.append(r + n - 1)
+            r += n
+        h = HostStep(B=len(batch.decode), T=T, nbt=max(1, R), bt_w=bt_w, bt_need=min(need, bt_w),
+                     n_rows=len(logit_rows), patch=patch, n_seg=R, owners=owners)
+        h.i64 = np.concatenate([tokens, positions, slots, np.asarray(logit_rows, dtype=np.int64)])
+        h.i32 = np.concatenate([bt.reshape(-1), tok_seg, seg.reshape(-1)])
+        h.stats = {"B": h.B, "T": T, "segments": R}
+        return h, sample_seqs
+
+    def build_host(self, batch: ScheduledBatch, want: dict | None = None) -> tuple[HostStep, list[Sequence]]:
+        """``want``: {seq_id: row offsets within the sequence's portion of this step} — return logits for exactly
+        these rows instead of one sampling row per sequence that reaches its end (trace replay).
+
+        All host-side work of a step: token/slot/page-table packing and attention work-item planning. The result
         is a few numpy arrays + scalars — what a TP leader broadcasts to its followers (``engine/tp_worker.py``).
 
         Decode rows are reordered so that every cascade group (rows sharing a KV prefix of at least
         ``cascade_min_prefix`` tokens, ``prefix_groups``) is contiguous: each group's prefix is attended once for all
         its rows by the tile kernel, the per-row suffixes by the decode kernel in pieces of about equal size."""
+        if self.segments:
+            return self._build_host_segments(batch, want)
         dec = list(batch.decode)
         B = len(dec)
         pre = batch.prefill
@@ -566,6 +645,7 @@ class ModelRunner:
         sample_seqs: list[Sequence] = []
         logit_rows: list[int] = []
         patch = []
+        owners: list = []
         for i, s in enumerate(dec):
             p = s.total_len - 1
             t = s.token_at(p)
@@ -575,8 +655,12 @@ class ModelRunner:
             positions[i] = p
             q_limit[i] = p
             self.kvm.fill_slots(s.seq_id, p, p + 1, slots, i)
-            sample_seqs.append(s)
-            logit_rows.append(i)
+            if want is None:
+                sample_seqs.append(s)
+                logit_rows.append(i)
+            elif want.get(s.seq_id):
+                logit_rows.append(i)
+                owners.append((s.seq_id, 0))
         tiles = []
         r = B
         for j, (s, a, b) in enumerate(pre):
@@ -589,7 +673,10 @@ class ModelRunner:
             for t0 in range(0, n, self.tile):
                 cnt = min(self.tile, n - t0)
                 tiles.append((r + t0 - B, cnt, bt_row, a + t0 + cnt, b))
-            if b == s.total_len:
+            if want is not None:
+                logit_rows += [r + o for o in want.get(s.seq_id, ())]
+                owners += [(s.seq_id, o) for o in want.get(s.seq_id, ())]
+            elif b == s.total_len:
                 sample_seqs.append(s)
                 logit_rows.append(r + n - 1)
             r += n
@@ -599,7 +686,8 @@ class ModelRunner:
             slots[T_real:] = -1
             q_limit[T_real:] = 0
         # ---- decode metadata (+ cascade over each group's shared prefix)
-        h = HostStep(B=B, T=T, nbt=nbt, bt_w=bt_w, bt_need=min(need, bt_w), n_rows=len(logit_rows), patch=patch)
+        h = HostStep(B=B, T=T, nbt=nbt, bt_w=bt_w, bt_need=min(need, bt_w), n_rows=len(logit_rows), patch=patch,
+                     owners=owners)
         i32_parts = [bt.reshape(-1), q_limit]
         # new-turn prefill chunks whose block table starts with a cascade group's prefix pages (the ~18k shared
         # system prompt every new turn of a thread re-attends): their tokens join the group's prefix pass — one read
@@ -750,6 +838,16 @@ class ModelRunner:
         B, T, nbt = h.B, h.T, h.nbt
         t_tokens, t_pos, t_slots = d64[0:T], d64[T:2 * T], d64[2 * T:3 * T]
         t_rows = d64[3 * T:3 * T + h.n_rows]
+        if h.n_seg:
+            from kafka_llm_service_amd.models.budurax import SegMeta
+
+            n_bt = nbt * h.bt_w
+            sm = SegMeta(T, h.n_seg, d32[n_bt + T:n_bt + T + 4 * h.n_seg].view(h.n_seg, 4), d32[n_bt:n_bt + T],
+                         d32[:n_bt].view(nbt, h.bt_w))
+            if h.n_late:
+                L, n = h.late_off, h.n_late
+                t_tokens.index_copy_(0, d64[L:L + n], self.tok_buf.index_select(0, d64[L + n:L + 2 * n]))
+            return StepInput(t_tokens, t_pos, t_slots, sm, t_rows)
         meta = AttnMeta(num_decode=B, num_tokens=T, scale=self.model.scale, variant=self.variant)
         o = 0
         n_bt = nbt * h.bt_w
@@ -969,6 +1067,16 @@ class ModelRunner:
             toks = self.sample_device(logits, sp)
             self.tok_buf[:toks.shape[0]].copy_(toks)
         return toks
+
+    @torch.inference_mode()
+    def forward_logits(self, host: HostStep, layers_out: list | None = None) -> torch.Tensor:
+        """One step without sampling: the logits of the plan's logit rows (trace replay; ``layers_out`` as
+        BuduraxLM.forward)."""
+        self.stager.begin()
+        inp = self.to_device(host)
+        if layers_out is not None:
+            return self.model.forward(inp, self.k_caches, self.v_caches, layers_out=layers_out)
+        return self.model.forward(inp, self.k_caches, self.v_caches)
 
     def collect(self, h: "Launched") -> list[int]:
         if h.event is not None:

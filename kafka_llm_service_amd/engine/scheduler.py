@@ -81,9 +81,12 @@ class NeedSync(Exception):
 
 
 class Scheduler:
-    def __init__(self, cfg: SchedulerConfig, kv):
+    def __init__(self, cfg: SchedulerConfig, kv, slots=None):
         self.cfg = cfg
         self.kv = kv
+        # runtime.StateSlots of a model with per-sequence recurrent state: a sequence holds one slot from admission
+        # until it finishes or is preempted (recompute restarts it from position 0, where state is zero by definition)
+        self.slots = slots
         self.page = kv.page
         self.waiting: deque[Sequence] = deque()
         self.running: list[Sequence] = []
@@ -110,6 +113,8 @@ class Scheduler:
 
     def _evict(self, seq: Sequence) -> None:
         self.kv.free_sequence(seq.seq_id)
+        if self.slots is not None:
+            self.slots.release(seq.seq_id)
         self.running.remove(seq)
         seq.status = SeqStatus.WAITING
         seq.num_computed = 0
@@ -129,6 +134,42 @@ class Scheduler:
                 pass
         if self.kv.has_seq(seq.seq_id):
             self.kv.free_sequence(seq.seq_id)
+        if self.slots is not None:
+            self.slots.release(seq.seq_id)
+
+    def replay(self, portions: list[tuple[Sequence, int]]) -> ScheduledBatch:
+        """A batch with caller-chosen portions (trace replay): the next ``n`` tokens of each listed sequence, in the
+        given order, admitting a sequence at its first portion. The same bookkeeping as ``schedule`` — pages, state
+        slots, the running list — without its policy; raises when the pool cannot hold a portion (a replay never
+        preempts)."""
+        batch = ScheduledBatch()
+        for seq, n in portions:
+            if n < 1 or seq.num_computed + n > seq.total_len:
+                raise ValueError(f"request {seq.request_id}: portion of {n} tokens at {seq.num_computed} of "
+                                 f"{seq.total_len}")
+            if seq.status == SeqStatus.WAITING:
+                if len(self.running) >= self.cfg.max_num_seqs:
+                    raise RuntimeError("more live requests than max_num_seqs")
+                cached = self.kv.add_sequence(seq.seq_id, seq.all_ids())
+                if self.slots is not None and self.slots.acquire(seq.seq_id) < 0:
+                    self.kv.free_sequence(seq.seq_id)
+                    raise RuntimeError("no free state slot")
+                try:
+                    self.waiting.remove(seq)
+                except ValueError:
+                    pass
+                seq.num_cached = seq.num_computed = cached
+                seq.status = SeqStatus.RUNNING
+                self.running.append(seq)
+                n = min(n, seq.total_len - cached) if cached else n
+            a, b = seq.num_computed, seq.num_computed + n
+            if not self.kv.ensure_capacity(seq.seq_id, b):
+                raise RuntimeError(f"KV pool exhausted at request {seq.request_id} ({b} tokens)")
+            if n == 1 and b == seq.total_len:
+                batch.decode.append(seq)
+            else:
+                batch.prefill.append((seq, a, b))
+        return batch
 
     @staticmethod
     def _grammar_plannable(seq: Sequence) -> bool:
@@ -211,6 +252,9 @@ class Scheduler:
                 break
             if not self.kv.ensure_capacity(seq.seq_id, end):
                 self.kv.free_sequence(seq.seq_id)
+                break
+            if self.slots is not None and self.slots.acquire(seq.seq_id) < 0:
+                self.kv.free_sequence(seq.seq_id)  # every state slot is held: wait for a sequence to finish
                 break
             cost += c
             admitted += 1

@@ -98,12 +98,54 @@ PRESETS: dict[str, ModelConfig] = {
 }
 
 
-def get_config(name: str) -> ModelConfig:
+def _budurax(width: int, heads: int, n_layers: int, vocab: int, ff: int, attn_every: int = 3) -> dict:
+    """A Budurax config dict at transformer-like sizes: 128-dim heads with a 64-dim rotary part, latent rank 4 x the
+    head size, every ``attn_every``-th layer latent attention (later ones borrow the first's cache), the rest Mamba-2."""
+    rot = {"base": 500000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}
+    layers = []
+    for i in range(n_layers):
+        if i % attn_every == 0:
+            m = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "rot": rot,
+                 "scale": (128 + 64) ** -0.5}
+            if i:
+                m["kv_from"] = 0
+            layers.append({"type": "latent_attention", "mixer": m, "mlp": {"kind": "dense", "ff": ff}})
+        else:
+            layers.append({"type": "mamba2", "mixer": {"heads": 2 * width // 64, "vdim": 64, "state": 128, "groups": 8,
+                                                       "norm_groups": 8, "conv": 4},
+                           "mlp": {"kind": "dense", "ff": ff}})
+    return {"architecture": "Budurax", "vocab": vocab, "width": width, "layers": layers, "norm": {"eps": 1e-6},
+            "token_side": {"dim": 64}}
+
+
+BUDURAX_PRESETS: dict[str, dict] = {
+    # sizes of the Llama presets below (same width, heads, depth, vocabulary and feed-forward), random init
+    "budurax-8b-shape": _budurax(4096, 32, 32, 128256, 14336),
+    "budurax-small": _budurax(1024, 16, 4, 128256, 3584),
+    "budurax-tiny": _budurax(512, 8, 3, 32000, 1024),
+}
+
+
+def _from_json(path: Path):
+    """A config.json names its model class: ``"architecture": "Budurax"`` (models/budurax.py), else HF Llama / Mixtral."""
+    c = json.loads(path.read_text())
+    if str(c.get("architecture", "")).lower() == "budurax":
+        from kafka_llm_service_amd.models.budurax import BuduraxConfig
+
+        return BuduraxConfig.from_dict(c, name=path.parent.name)
+    return ModelConfig.from_hf(path)
+
+
+def get_config(name: str):
     if name in PRESETS:
         return PRESETS[name]
+    if name in BUDURAX_PRESETS:
+        from kafka_llm_service_amd.models.budurax import BuduraxConfig
+
+        return BuduraxConfig.from_dict(BUDURAX_PRESETS[name], name=name)
     p = Path(name)
     if p.is_dir() and (p / "config.json").exists():
-        return ModelConfig.from_hf(p / "config.json")
+        return _from_json(p / "config.json")
     if p.suffix == ".json" and p.exists():
-        return ModelConfig.from_hf(p)
+        return _from_json(p)
     raise KeyError(f"unknown model {name!r}; presets: {sorted(PRESETS)}")

@@ -270,8 +270,19 @@ def save_safetensors(model: TransformerLM, path: str | Path) -> None:
 
 
 def build_model(cfg: ModelConfig, device, tp: int = 1, tp_rank: int = 0, seed: int = 0, weights: str | None = None,
-                max_positions: int | None = None, dp_attention: tuple[int, int] | None = None) -> TransformerLM:
-    """``dp_attention = (ep, ep_rank)``: whole attention on this rank, experts sharded over the EP group."""
+                max_positions: int | None = None, dp_attention: tuple[int, int] | None = None, dtype=None):
+    """``dp_attention = (ep, ep_rank)``: whole attention on this rank, experts sharded over the EP group.
+    The model class follows ``cfg.arch`` (MODEL_CLASSES)."""
+    if cfg.arch == "budurax":
+        from kafka_llm_service_amd.models import budurax as bx
+
+        model = bx.BuduraxLM(cfg, device, dtype=dtype or torch.bfloat16, tp=tp, tp_rank=tp_rank,
+                             max_positions=max_positions)
+        if weights:
+            return bx.load_checkpoint(model, weights)
+        return model.load_tensors(bx.random_tensors(cfg, seed))
+    if dtype not in (None, torch.bfloat16):
+        raise ValueError(f"{cfg.arch} models run in bfloat16 only")
     model = TransformerLM(cfg, device, tp=tp, tp_rank=tp_rank, max_positions=max_positions)
     if dp_attention is not None:
         model.enable_dp_attention(*dp_attention)

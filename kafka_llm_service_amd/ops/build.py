@@ -17,7 +17,9 @@ CSRC = HERE / "csrc"
 OUT = HERE / "_kafka_ops.so"
 
 HIP_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-munsafe-fp-atomics",
-             "-fgpu-flush-denormals-to-zero", "-Wno-unused-result"]
+             "-fgpu-flush-denormals-to-zero", "-Wno-unused-result",
+             # no packed fp32 arithmetic: the compiler's v_pk_*_f32 forms are kept out of every kernel
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
 def build(verbose: bool = False) -> Path:

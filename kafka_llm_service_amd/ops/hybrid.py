@@ -1,0 +1,124 @@
+"""Ops of the hybrid decoder family (layer norm, token shift, latent attention, Mamba-2, depth average): GPU tensors
+run the HIP kernels of ``csrc/hybrid.hip``, CPU tensors the fp32 references of ``hybrid_reference.py``.
+
+Activations are bf16 or fp32 (the model's dtype, the kernels are built for both); the residual stream, recurrent
+state, norms, softmax and every gate of a recurrence are fp32 in both. A step's rows are described by ``seg`` int32
+[R, 4] = (first row, rows, first position, state slot) and ``tok_seg`` int32 [T] (see hybrid_reference.py).
+"""
+from __future__ import annotations
+
+import torch
+
+from . import hybrid_reference as ref
+from ._ext import ext
+
+SCAN_MAX_TAPS = 8
+
+
+def _gpu(t: torch.Tensor) -> bool:
+    return t.is_cuda
+
+
+def ln_shift(x, w, b, eps, out, mu=None, tok_seg=None, seg=None, state=None, last=None) -> None:
+    """out = layer_norm(x) (x fp32 [T, d]); with ``mu`` each row is then moved towards the previous row's normed
+    value (the slot's ``state`` row for a segment's first row) by mu, and every segment's last normed row lands in
+    ``last`` [R, d] (``scatter_rows`` stores it once all rows have read the old state)."""
+    if _gpu(x):
+        ext().hy_ln_shift(x, w, b, float(eps), out, mu, tok_seg, seg, state, last)
+    else:
+        ref.ln_shift(x, w, b, eps, out, mu, tok_seg, seg, state, last)
+
+
+def scatter_rows(dst, seg, src) -> None:
+    """dst[seg[r].slot] = src[r]."""
+    if _gpu(dst):
+        ext().hy_scatter_rows(dst, seg, src)
+    else:
+        ref.scatter_rows(dst, seg, src)
+
+
+def add_ln(x, y, w, b, eps, out2=None, w2=None, b2=None) -> None:
+    """x += layer_norm(y; w, b) in place (x fp32); with ``out2`` also out2 = layer_norm(x; w2, b2), or the new x in
+    out2's dtype when no second norm is given."""
+    if _gpu(x):
+        ext().hy_add_ln(x, y, w, b, float(eps), out2, w2, b2)
+    else:
+        ref.add_ln(x, y, w, b, eps, out2, w2, b2)
+
+
+def gelu_mul(gu, out) -> None:
+    """out = gelu_tanh(gu[:, :F]) * gu[:, F:]."""
+    if _gpu(gu):
+        ext().hy_gelu_mul(gu, out)
+    else:
+        ref.gelu_mul(gu, out)
+
+
+def side_gate(sg, tokens, side_embed, col0: int, out) -> None:
+    """out = gelu_tanh(sg) * side_embed[token, col0 : col0 + dim]."""
+    if _gpu(sg):
+        ext().hy_side_gate(sg, tokens, side_embed, int(col0), out)
+    else:
+        ref.side_gate(sg, tokens, side_embed, col0, out)
+
+
+def side_dwa(x, y, side_w, eps, stack, layer: int, dwa) -> None:
+    """x += y / rms(y) * side_w (when y is given); stack[layer + 1] = x; with ``dwa`` x = sum_j dwa[j] stack[j]."""
+    if _gpu(x):
+        ext().hy_side_dwa(x, y, side_w, float(eps), stack, int(layer), dwa)
+    else:
+        ref.side_dwa(x, y, side_w, eps, stack, layer, dwa)
+
+
+def latent_prep(qgd, H, dim, rd, R, dkv_off, dkv_w, eps, positions, cos_sin, rot_dims, cache, slot_mapping,
+                q_rot) -> None:
+    if _gpu(qgd):
+        ext().hy_latent_prep(qgd, int(H), int(dim), int(rd), int(R), int(dkv_off), dkv_w, float(eps), positions,
+                             cos_sin, int(rot_dims), cache, slot_mapping, q_rot)
+    else:
+        ref.latent_prep(qgd, H, dim, rd, R, dkv_off, dkv_w, eps, positions, cos_sin, rot_dims, cache, slot_mapping,
+                        q_rot)
+
+
+def latent_attn(q_lat, q_rot, cache, block_tables, tok_seg, seg, positions, scale, out) -> None:
+    """Causal softmax attention of every row's heads over its sequence's cached [latent | rotated key] rows."""
+    if _gpu(q_lat):
+        ext().hy_latent_attn(q_lat, q_rot, cache, block_tables, tok_seg, positions, float(scale), out)
+    else:
+        ref.latent_attn(q_lat, q_rot, cache, block_tables, tok_seg, seg, positions, scale, out)
+
+
+def sigmoid_mul(a, g, out) -> None:
+    if _gpu(a):
+        ext().hy_sigmoid_mul(a, g, out)
+    else:
+        ref.sigmoid_mul(a, g, out)
+
+
+def conv_silu(proj, c0: int, w, b, tok_seg, seg, state, out) -> None:
+    """Causal per-channel convolution + silu over columns [c0, c0 + C) of ``proj``; ``state`` [slots, taps - 1, C]
+    holds each sequence's last raw inputs and is advanced."""
+    if w.shape[1] > SCAN_MAX_TAPS:
+        raise ValueError(f"short convolution of {w.shape[1]} taps (at most {SCAN_MAX_TAPS})")
+    if _gpu(proj):
+        ext().hy_conv_silu(proj, int(c0), w, b, tok_seg, seg, state, out)
+    else:
+        ref.conv_silu(proj, c0, w, b, tok_seg, seg, state, out)
+
+
+def ssm_scan(xbc, proj, dt_off: int, dt_bias, A_log, D, heads, P, N, G, tok_seg, seg, state, y) -> None:
+    """Mamba-2 recurrence per (segment, head): S <- exp(-exp(A_log) dt) S + dt B x^T, y = S^T C + D x, with
+    dt = softplus(raw dt + bias); fp32 state [slots, heads, N, P] read (unless the segment starts at 0) and left."""
+    if _gpu(xbc):
+        ext().hy_ssm_scan(xbc, proj, int(dt_off), dt_bias, A_log, D, int(heads), int(P), int(N), int(G), seg, state,
+                          y)
+    else:
+        ref.ssm_scan(xbc, proj, dt_off, dt_bias, A_log, D, heads, P, N, G, tok_seg, seg, state, y)
+
+
+def gated_norm(y, proj, w, groups: int, eps, out) -> None:
+    """out = group_rms_norm(y * silu(proj[:, :inner])) * w, the norm over ``groups`` equal parts of a row."""
+    if _gpu(y):
+        ext().hy_gated_norm(y, proj, w, int(groups), float(eps), out)
+    else:
+        ref.gated_norm(y, proj, w, groups, eps, out)

@@ -24,3 +24,8 @@ def native():
 
 def KVManager(num_blocks: int, page: int = 16, prefix_cache: bool = True, run: int = 1):
     return native().KVManager(num_blocks, page, prefix_cache, run)
+
+
+def StateSlots(num_slots: int):
+    """Pool of per-sequence recurrent-state slots (runtime/csrc/state_slots.cpp)."""
+    return native().StateSlots(num_slots)
