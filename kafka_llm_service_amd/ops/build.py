@@ -29,7 +29,7 @@ def build(verbose: bool = False) -> Path:
                   "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=_kafka_ops", "-DTORCH_API_INCLUDE_EXTENSION_H",
                   f"-I{ROCM / 'include'}", f"-I{python_include()}", *[f"-I{p}" for p in tincs],
                   "-Wno-deprecated-declarations"]
-    units.append(Unit(CSRC / "bindings.cpp", "g++", bind_flags))
+    units += [Unit(CSRC / n, "g++", bind_flags) for n in ("bindings.cpp", "hybrid_bindings.cpp")]
     tlib = troot / "lib"
     link = [f"--offload-arch={ARCH}", f"-L{tlib}", "-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu", "-ltorch_hip",
             "-ltorch_python", f"-Wl,-rpath,{tlib}", "-Wl,--no-undefined" if False else "-Wl,-O1"]

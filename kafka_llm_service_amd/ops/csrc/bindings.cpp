@@ -988,8 +988,11 @@ static void ep_combine(at::Tensor back, at::Tensor slot_map, at::Tensor topk_w, 
                                     (int)n_own, k, d, bptr(out), out.stride(0), cur_stream()));
 }
 
+void kafka_bind_hybrid(pybind11::module_& m);  // hybrid_bindings.cpp
+
 PYBIND11_MODULE(_kafka_ops, m) {
   m.doc() = "kafka_llm_service_amd CDNA4 (gfx950) HIP kernels";
+  kafka_bind_hybrid(m);
   m.def("rmsnorm", &rmsnorm);
   m.def("fused_add_rmsnorm", &fused_add_rmsnorm);
   m.def("silu_mul", &silu_mul);

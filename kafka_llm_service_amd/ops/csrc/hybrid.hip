@@ -1,0 +1,651 @@
+// Kernels of the hybrid decoder family (latent attention + Mamba-2 layers, layer norms before and after every
+// sublayer, token shift, per-layer token input, depth average) for gfx950.
+//
+// Every kernel is built for bf16 and for fp32 activations (template AT); the residual stream, the recurrent state,
+// every norm's statistics, softmax, rotary products and the recurrence's gates are fp32 in both. Sizes are run-time
+// values with no alignment assumptions (channel counts, head sizes and ranks come from the model's config), so rows
+// are walked with scalar, lane-consecutive (coalesced) accesses.
+//
+// A step's rows are described by segments: seg[r] = (first row, rows, first position, state slot), one per sequence
+// in the step, and tok_seg[t] = the segment of row t. A segment whose first position is 0 has zero state: its slot is
+// written, never read, so reused slots need no clearing.
+//
+//   ln_shift        layer norm (weight + bias) of the fp32 stream -> AT; with a shift vector each row is moved towards
+//                   the previous row's normed value (the slot's state for a segment's first row) - the previous row
+//                   is re-normed by the same workgroup, nothing is exchanged between workgroups
+//   add_ln          x += layer_norm(y) and, in the same pass over the row, the next sublayer's pre-norm of the new x
+//   side_dwa        x += unit_rms(y) * w, push x on the depth stack, x = sum_j a_j stack_j
+//   latent_prep     RMS norm of the latent + rotary on the shared key part -> paged cache row; rotary on the query parts
+//   latent_attn     all heads of a row against the row's cached [latent | rotary key] rows: one wave per (row, 4
+//                   heads), the 64 lanes across the row's dimensions, online softmax, the value pass reusing the key
+//                   registers (the values ARE the latent part of the key row)
+//   conv_silu       causal short convolution + silu with a per-slot tail of raw inputs
+//   ssm_scan        the state-space recurrence, one workgroup per (segment, head), state in registers, B / C / x / dt
+//                   of 8 tokens staged through LDS
+//   gated_norm      y * silu(z), RMS norm in groups, weight
+#include "common.h"
+
+namespace kafka {
+namespace hy {
+
+template <typename T>
+__device__ __forceinline__ float ldf(const T* p) { return (float)(*p); }
+template <typename T>
+__device__ __forceinline__ void stf(T* p, float v) { *p = (T)v; }
+
+__device__ __forceinline__ float gelu_tanh(float z) {
+  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+__device__ __forceinline__ float sigmoidf(float z) { return 1.0f / (1.0f + expf(-z)); }
+__device__ __forceinline__ float inv_sqrt(float v) { return 1.0f / sqrtf(v); }
+
+constexpr int NT = 256;
+
+// mean and 1 / sqrt(var + eps) of an fp32 or AT row
+template <typename XT>
+__device__ __forceinline__ void row_stats(const XT* __restrict__ r, int d, float eps, float* red, float& mean,
+                                          float& rstd) {
+  float s = 0.f;
+  for (int i = threadIdx.x; i < d; i += NT) s += ldf(r + i);
+  mean = block_sum<NT>(s, red) / (float)d;
+  float v = 0.f;
+  for (int i = threadIdx.x; i < d; i += NT) {
+    const float c = ldf(r + i) - mean;
+    v += c * c;
+  }
+  rstd = inv_sqrt(block_sum<NT>(v, red) / (float)d + eps);
+}
+
+template <typename AT>
+__global__ __launch_bounds__(NT) void ln_shift_kernel(const float* __restrict__ x, int64_t xs, const AT* __restrict__ w,
+                                                      const AT* __restrict__ b, float eps, AT* __restrict__ out,
+                                                      int64_t os, int d, const AT* __restrict__ mu,
+                                                      const int* __restrict__ tok_seg, const int* __restrict__ seg,
+                                                      const float* __restrict__ state, float* __restrict__ last) {
+  __shared__ float red[NT / 64];
+  const int64_t t = blockIdx.x;
+  const float* xr = x + t * xs;
+  float mean, rstd;
+  row_stats(xr, d, eps, red, mean, rstd);
+  if (mu == nullptr) {
+    for (int i = threadIdx.x; i < d; i += NT) stf(out + t * os + i, (xr[i] - mean) * rstd * ldf(w + i) + ldf(b + i));
+    return;
+  }
+  const int sg = tok_seg[t];
+  const int q0 = seg[4 * sg], n = seg[4 * sg + 1], p0 = seg[4 * sg + 2], slot = seg[4 * sg + 3];
+  const bool first = (t == q0), is_last = (t == q0 + n - 1);
+  float mean2 = 0.f, rstd2 = 0.f;
+  const float* xp = xr - xs;
+  if (!first) row_stats(xp, d, eps, red, mean2, rstd2);  // (uniform per workgroup)
+  for (int i = threadIdx.x; i < d; i += NT) {
+    const float wi = ldf(w + i), bi = ldf(b + i);
+    const float h = (xr[i] - mean) * rstd * wi + bi;
+    float prev;
+    if (first)
+      prev = p0 > 0 ? state[(int64_t)slot * d + i] : 0.f;
+    else
+      prev = (xp[i] - mean2) * rstd2 * wi + bi;
+    stf(out + t * os + i, h + (prev - h) * ldf(mu + i));
+    if (is_last) last[(int64_t)sg * d + i] = h;
+  }
+}
+
+__global__ void scatter_rows_kernel(float* __restrict__ dst, const int* __restrict__ seg, const float* __restrict__ src,
+                                    int d) {
+  const int r = blockIdx.x;
+  const int slot = seg[4 * r + 3];
+  for (int i = threadIdx.x; i < d; i += blockDim.x) dst[(int64_t)slot * d + i] = src[(int64_t)r * d + i];
+}
+
+// x += ln(y; w, b); MODE 1: out2 = ln(x_new; w2, b2); MODE 2: out2 = x_new (cast)
+template <typename AT, int MODE>
+__global__ __launch_bounds__(NT) void add_ln_kernel(float* __restrict__ x, int64_t xs, const AT* __restrict__ y,
+                                                    int64_t ys, const AT* __restrict__ w, const AT* __restrict__ b,
+                                                    float eps, int d, AT* __restrict__ out2, int64_t os,
+                                                    const AT* __restrict__ w2, const AT* __restrict__ b2) {
+  __shared__ float red[NT / 64];
+  const int64_t t = blockIdx.x;
+  const AT* yr = y + t * ys;
+  float* xr = x + t * xs;
+  float mean, rstd;
+  row_stats(yr, d, eps, red, mean, rstd);
+  for (int i = threadIdx.x; i < d; i += NT) {
+    const float v = xr[i] + ((ldf(yr + i) - mean) * rstd * ldf(w + i) + ldf(b + i));
+    xr[i] = v;  // re-read below by the same thread only
+    if constexpr (MODE == 2) stf(out2 + t * os + i, v);
+  }
+  if constexpr (MODE == 1) {
+    float m2, r2;
+    row_stats(xr, d, eps, red, m2, r2);
+    for (int i = threadIdx.x; i < d; i += NT)
+      stf(out2 + t * os + i, (xr[i] - m2) * r2 * ldf(w2 + i) + ldf(b2 + i));
+  }
+}
+
+template <typename AT>
+__global__ void gelu_mul_kernel(const AT* __restrict__ gu, int64_t gs, AT* __restrict__ out, int64_t T, int F) {
+  const int64_t n = T * F;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t t = i / F;
+    const int f = (int)(i - t * F);
+    stf(out + i, gelu_tanh(ldf(gu + t * gs + f)) * ldf(gu + t * gs + F + f));
+  }
+}
+
+template <typename AT>
+__global__ void side_gate_kernel(const AT* __restrict__ sg, int64_t ss, const int64_t* __restrict__ tokens,
+                                 const AT* __restrict__ emb, int64_t es, int col0, AT* __restrict__ out, int64_t T,
+                                 int dim) {
+  const int64_t n = T * dim;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t t = i / dim;
+    const int j = (int)(i - t * dim);
+    stf(out + i, gelu_tanh(ldf(sg + t * ss + j)) * ldf(emb + tokens[t] * es + col0 + j));
+  }
+}
+
+template <typename AT>
+__global__ __launch_bounds__(NT) void side_dwa_kernel(float* __restrict__ x, const AT* __restrict__ y, int64_t ys,
+                                                      const AT* __restrict__ sw, float eps, float* __restrict__ stack,
+                                                      int layer, const float* __restrict__ dwa, int64_t T, int d) {
+  __shared__ float red[NT / 64];
+  const int64_t t = blockIdx.x;
+  float* xr = x + t * d;
+  float r = 0.f;
+  if (y != nullptr) {
+    float s = 0.f;
+    for (int i = threadIdx.x; i < d; i += NT) {
+      const float v = ldf(y + t * ys + i);
+      s += v * v;
+    }
+    r = inv_sqrt(block_sum<NT>(s, red) / (float)d + eps);
+  }
+  const int64_t plane = T * d;
+  for (int i = threadIdx.x; i < d; i += NT) {
+    float v = xr[i];
+    if (y != nullptr) v += ldf(y + t * ys + i) * r * ldf(sw + i);
+    if (stack != nullptr) {
+      stack[(int64_t)(layer + 1) * plane + t * d + i] = v;
+      if (dwa != nullptr) {
+        float a = 0.f;
+        for (int j = 0; j <= layer; ++j) a += dwa[j] * stack[(int64_t)j * plane + t * d + i];
+        v = a + dwa[layer + 1] * v;
+      }
+    }
+    xr[i] = v;
+  }
+}
+
+// rotate-half rotary of one element j of a `rd`-long vector v (first `dims` entries rotate, the rest pass)
+template <typename AT>
+__device__ __forceinline__ float rot_elem(const AT* v, int j, int dims, const float* cs) {
+  const int half = dims >> 1;
+  const float a = ldf(v + j);
+  if (j >= dims) return a;
+  if (j < half) return a * cs[j] - ldf(v + j + half) * cs[half + j];
+  return a * cs[j - half] + ldf(v + j - half) * cs[j];  // cs[half + (j - half)] = sin
+}
+
+template <typename AT>
+__global__ __launch_bounds__(NT) void latent_prep_kernel(const AT* __restrict__ qgd, int64_t qs, int H, int dim, int rd,
+                                                         int R, int dkv_off, const AT* __restrict__ dkv_w, float eps,
+                                                         const int64_t* __restrict__ positions,
+                                                         const float* __restrict__ cos_sin, int dims,
+                                                         AT* __restrict__ cache, const int64_t* __restrict__ slots,
+                                                         AT* __restrict__ q_rot) {
+  __shared__ float red[NT / 64];
+  const int64_t t = blockIdx.x;
+  const AT* row = qgd + t * qs;
+  const float* cs = cos_sin + positions[t] * dims;
+  for (int i = threadIdx.x; i < H * rd; i += NT) {
+    const int h = i / rd, j = i - h * rd;
+    stf(q_rot + (t * H + h) * rd + j, rot_elem(row + (int64_t)h * (dim + rd) + dim, j, dims, cs));
+  }
+  if (dkv_off < 0) return;
+  const int64_t slot = slots[t];
+  const AT* lat = row + dkv_off;
+  float s = 0.f;
+  for (int i = threadIdx.x; i < R; i += NT) {
+    const float v = ldf(lat + i);
+    s += v * v;
+  }
+  const float r = inv_sqrt(block_sum<NT>(s, red) / (float)R + eps);
+  if (slot < 0) return;
+  AT* dst = cache + slot * (R + rd);
+  for (int i = threadIdx.x; i < R; i += NT) stf(dst + i, ldf(lat + i) * r * ldf(dkv_w + i));
+  for (int j = threadIdx.x; j < rd; j += NT) stf(dst + R + j, rot_elem(lat + R, j, dims, cs));
+}
+
+template <typename AT>
+__global__ void sigmoid_mul_kernel(const AT* __restrict__ a, int64_t a_h, int64_t a_t, const AT* __restrict__ g,
+                                   int64_t gs, AT* __restrict__ out, int64_t T, int H, int vd) {
+  const int64_t n = T * H * vd;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t t = i / (H * vd);
+    const int c = (int)(i - t * H * vd);
+    const int h = c / vd, j = c - h * vd;
+    stf(out + i, ldf(a + h * a_h + t * a_t + j) * sigmoidf(ldf(g + t * gs + c)));
+  }
+}
+
+// ---- latent attention ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ float wave_allsum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+// One wave per (row t, group of RPW heads). Lane l holds dimensions l, l + 64, ... of the query rows, of the key row
+// being visited and of the output accumulators; a key row is loaded once for the wave's heads, and its latent part
+// is also the value row. Keys are visited in order 0 .. position, KB at a time, whatever the step's batch: a row's
+// result does not depend on what else runs.
+template <typename AT, int MAXC, int RPW, int KB>
+__global__ __launch_bounds__(256) void latent_attn_kernel(const AT* __restrict__ q_lat, int64_t ql_h, int64_t ql_t,
+                                                          const AT* __restrict__ q_rot, int64_t qr_t, int64_t qr_h,
+                                                          const AT* __restrict__ cache, int page, int R, int rd,
+                                                          const int* __restrict__ bt, int bt_stride,
+                                                          const int* __restrict__ tok_seg,
+                                                          const int64_t* __restrict__ positions, float scale_log2e,
+                                                          AT* __restrict__ out, int64_t o_h, int64_t o_t, int T, int H,
+                                                          int n_hg) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t task = (int64_t)blockIdx.x * 4 + wave;
+  if (task >= (int64_t)T * n_hg) return;
+  const int t = (int)(task / n_hg), hg = (int)(task - (int64_t)t * n_hg);
+  const int h0 = hg * RPW;
+  const int nh = min(RPW, H - h0);
+  const int Dk = R + rd;
+  float q[RPW][MAXC], acc[RPW][MAXC], m[RPW], l[RPW];
+#pragma unroll
+  for (int r = 0; r < RPW; ++r) {
+    m[r] = -INFINITY;
+    l[r] = 0.f;
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+      const int dim = lane + 64 * c;
+      float v = 0.f;
+      if (r < nh && dim < Dk)
+        v = dim < R ? ldf(q_lat + (int64_t)(h0 + r) * ql_h + (int64_t)t * ql_t + dim)
+                    : ldf(q_rot + (int64_t)t * qr_t + (int64_t)(h0 + r) * qr_h + (dim - R));
+      q[r][c] = v * scale_log2e;
+      acc[r][c] = 0.f;
+    }
+  }
+  const int nkeys = (int)positions[t] + 1;
+  const int* btr = bt + (int64_t)tok_seg[t] * bt_stride;
+  for (int j0 = 0; j0 < nkeys; j0 += KB) {
+    float k[KB][MAXC];
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) {
+      const int j = min(j0 + kb, nkeys - 1);
+      const int64_t slot = (int64_t)btr[j / page] * page + (j % page);
+      const AT* kr = cache + slot * Dk;
+#pragma unroll
+      for (int c = 0; c < MAXC; ++c) {
+        const int dim = lane + 64 * c;
+        k[kb][c] = dim < Dk ? ldf(kr + dim) : 0.f;
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) {
+      if (r < nh) {
+        float s[KB];
+        float mn = m[r];
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+          float part = 0.f;
+#pragma unroll
+          for (int c = 0; c < MAXC; ++c) part += q[r][c] * k[kb][c];
+          s[kb] = wave_allsum(part);
+          if (j0 + kb >= nkeys) s[kb] = -INFINITY;
+          mn = fmaxf(mn, s[kb]);
+        }
+        const float corr = fast_exp2(m[r] - mn);  // 0 on the first block (m = -inf, mn finite)
+        float psum = 0.f;
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+          s[kb] = fast_exp2(s[kb] - mn);
+          psum += s[kb];
+        }
+        l[r] = l[r] * corr + psum;
+        m[r] = mn;
+#pragma unroll
+        for (int c = 0; c < MAXC; ++c) {
+          float a = acc[r][c] * corr;
+#pragma unroll
+          for (int kb = 0; kb < KB; ++kb) a += s[kb] * k[kb][c];
+          acc[r][c] = a;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < RPW; ++r) {
+    if (r < nh) {
+      const float inv = 1.0f / l[r];
+#pragma unroll
+      for (int c = 0; c < MAXC; ++c) {
+        const int dim = lane + 64 * c;
+        if (dim < R) stf(out + (int64_t)(h0 + r) * o_h + (int64_t)t * o_t + dim, acc[r][c] * inv);
+      }
+    }
+  }
+}
+
+// ---- Mamba-2 ---------------------------------------------------------------------------------------------------------
+template <typename AT>
+__global__ void conv_silu_kernel(const AT* __restrict__ proj, int64_t ps, int c0, const AT* __restrict__ w,
+                                 const AT* __restrict__ b, int C, int taps, const int* __restrict__ tok_seg,
+                                 const int* __restrict__ seg, const AT* __restrict__ state, AT* __restrict__ out,
+                                 int64_t T) {
+  const int64_t n = T * C;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t t = i / C;
+    const int c = (int)(i - t * C);
+    const int sg = tok_seg[t];
+    const int q0 = seg[4 * sg], p0 = seg[4 * sg + 2], slot = seg[4 * sg + 3];
+    float a = ldf(b + c);
+    for (int k = 0; k < taps; ++k) {
+      const int64_t src = t - (taps - 1 - k);
+      float u = 0.f;
+      if (src >= q0) {
+        u = ldf(proj + src * ps + c0 + c);
+      } else if (p0 > 0) {
+        const int si = taps - 1 + (int)(src - q0);  // the slot's tail holds the inputs before the segment
+        if (si >= 0) u = ldf(state + ((int64_t)slot * (taps - 1) + si) * C + c);
+      }
+      a += u * ldf(w + (int64_t)c * taps + k);
+    }
+    stf(out + i, a / (1.0f + expf(-a)));
+  }
+}
+
+// the slot's tail <- the last taps - 1 entries of (old tail ++ the segment's raw inputs); one thread per (segment,
+// channel) reads all it needs before it writes
+template <typename AT>
+__global__ void conv_state_kernel(const AT* __restrict__ proj, int64_t ps, int c0, int C, int taps,
+                                  const int* __restrict__ seg, AT* __restrict__ state, int R) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (int64_t)R * C) return;
+  const int r = (int)(i / C), c = (int)(i - (int64_t)r * C);
+  const int q0 = seg[4 * r], n = seg[4 * r + 1], p0 = seg[4 * r + 2], slot = seg[4 * r + 3];
+  AT* st = state + (int64_t)slot * (taps - 1) * C + c;
+  AT v[8];
+  for (int k = 0; k < taps - 1; ++k) {
+    const int at = n + k;  // index in (old tail ++ inputs)
+    if (at < taps - 1)
+      v[k] = p0 > 0 ? st[(int64_t)at * C] : (AT)0.f;
+    else
+      v[k] = proj[(int64_t)(q0 + at - (taps - 1)) * ps + c0 + c];
+  }
+  for (int k = 0; k < taps - 1; ++k) st[(int64_t)k * C] = v[k];
+}
+
+constexpr int SCAN_TB = 8;
+
+template <typename AT, int EPT>
+__global__ void ssm_scan_kernel(const AT* __restrict__ xbc, int64_t xs, const AT* __restrict__ proj, int64_t ps,
+                                int dt_off, const float* __restrict__ dt_bias, const float* __restrict__ A_log,
+                                const float* __restrict__ Dp, int heads, int P, int N, int G, int NG,
+                                const int* __restrict__ seg, float* __restrict__ state, float* __restrict__ y,
+                                int64_t ys) {
+  extern __shared__ float sm[];
+  const int sgi = blockIdx.x / heads, h = blockIdx.x - sgi * heads;
+  const int q0 = seg[4 * sgi], n = seg[4 * sgi + 1], p0 = seg[4 * sgi + 2], slot = seg[4 * sgi + 3];
+  const int tid = threadIdx.x, nthr = blockDim.x;
+  const int p = tid % P, g = tid / P;
+  const int grp = h / (heads / G);
+  const int inner = heads * P;
+  float S[EPT];
+  float* st = state + ((int64_t)slot * heads + h) * N * P;
+#pragma unroll
+  for (int k = 0; k < EPT; ++k) {
+    const int nn = g + k * NG;
+    S[k] = (p0 > 0 && nn < N) ? st[(int64_t)nn * P + p] : 0.f;
+  }
+  const float A = -expf(A_log[h]), bias = dt_bias[h], Dh = Dp[h];
+  float* Bs = sm;                    // [TB][N]  (dt * B)
+  float* Cs = Bs + SCAN_TB * N;      // [TB][N]
+  float* xv = Cs + SCAN_TB * N;      // [TB][P]
+  float* dts = xv + SCAN_TB * P;     // [TB]
+  float* dAs = dts + SCAN_TB;        // [TB]
+  float* yp = dAs + SCAN_TB;         // [TB][NG][P]
+  for (int t0 = 0; t0 < n; t0 += SCAN_TB) {
+    const int nt = min(SCAN_TB, n - t0);
+    if (tid < nt) {
+      const float raw = ldf(proj + (int64_t)(q0 + t0 + tid) * ps + dt_off + h) + bias;
+      const float dt = raw > 20.f ? raw : log1pf(expf(raw));  // softplus
+      dts[tid] = dt;
+      dAs[tid] = expf(A * dt);
+    }
+    __syncthreads();
+    for (int i = tid; i < nt * N; i += nthr) {
+      const int tt = i / N, nn = i - tt * N;
+      const AT* row = xbc + (int64_t)(q0 + t0 + tt) * xs + inner + grp * N + nn;
+      Bs[i] = dts[tt] * ldf(row);
+      Cs[i] = ldf(row + (int64_t)G * N);
+    }
+    for (int i = tid; i < nt * P; i += nthr) {
+      const int tt = i / P, pp = i - tt * P;
+      xv[i] = ldf(xbc + (int64_t)(q0 + t0 + tt) * xs + h * P + pp);
+    }
+    __syncthreads();
+    for (int tt = 0; tt < nt; ++tt) {
+      const float dA = dAs[tt], xp = xv[tt * P + p];
+      float a = 0.f;
+#pragma unroll
+      for (int k = 0; k < EPT; ++k) {
+        const int nn = g + k * NG;
+        if (nn < N) {
+          S[k] = dA * S[k] + Bs[tt * N + nn] * xp;
+          a += S[k] * Cs[tt * N + nn];
+        }
+      }
+      yp[(tt * NG + g) * P + p] = a;
+    }
+    __syncthreads();
+    for (int i = tid; i < nt * P; i += nthr) {
+      const int tt = i / P, pp = i - tt * P;
+      float s = 0.f;
+      for (int gg = 0; gg < NG; ++gg) s += yp[(tt * NG + gg) * P + pp];
+      y[(int64_t)(q0 + t0 + tt) * ys + h * P + pp] = s + Dh * xv[i];
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int k = 0; k < EPT; ++k) {
+    const int nn = g + k * NG;
+    if (nn < N) st[(int64_t)nn * P + p] = S[k];
+  }
+}
+
+template <typename AT>
+__global__ __launch_bounds__(NT) void gated_norm_kernel(const float* __restrict__ y, int64_t ys, const AT* __restrict__ z,
+                                                        int64_t zs, const AT* __restrict__ w, int gs, float eps,
+                                                        AT* __restrict__ out, int64_t os) {
+  __shared__ float red[NT / 64];
+  const int64_t t = blockIdx.x;
+  const int c0 = blockIdx.y * gs;
+  float s = 0.f;
+  for (int i = threadIdx.x; i < gs; i += NT) {
+    const float zv = ldf(z + t * zs + c0 + i);
+    const float v = y[t * ys + c0 + i] * (zv / (1.0f + expf(-zv)));
+    s += v * v;
+  }
+  const float r = inv_sqrt(block_sum<NT>(s, red) / (float)gs + eps);
+  for (int i = threadIdx.x; i < gs; i += NT) {
+    const float zv = ldf(z + t * zs + c0 + i);
+    const float v = y[t * ys + c0 + i] * (zv / (1.0f + expf(-zv)));
+    stf(out + t * os + c0 + i, v * r * ldf(w + c0 + i));
+  }
+}
+
+static inline int ew_grid(int64_t n) { return (int)std::min<int64_t>((n + 255) / 256, 65535 * 4); }
+
+}  // namespace hy
+}  // namespace kafka
+
+using namespace kafka::hy;
+
+#define DISPATCH_AT(f32, ...)             \
+  if (f32) {                              \
+    using AT = float;                     \
+    __VA_ARGS__;                          \
+  } else {                                \
+    using AT = bf16;                      \
+    __VA_ARGS__;                          \
+  }
+
+extern "C" {
+
+hipError_t kafka_hy_ln_shift(int f32, const float* x, int64_t xs, const void* w, const void* b, float eps, void* out,
+                             int64_t os, int T, int d, const void* mu, const int* tok_seg, const int* seg,
+                             const float* state, float* last, hipStream_t st) {
+  if (T <= 0) return hipSuccess;
+  DISPATCH_AT(f32, ln_shift_kernel<AT><<<T, NT, 0, st>>>(x, xs, (const AT*)w, (const AT*)b, eps, (AT*)out, os, d,
+                                                        (const AT*)mu, tok_seg, seg, state, last));
+  return hipGetLastError();
+}
+
+hipError_t kafka_hy_scatter_rows(float* dst, const int* seg, const float* src, int R, int d, hipStream_t st) {
+  if (R <= 0) return hipSuccess;
+  scatter_rows_kernel<<<R, 256, 0, st>>>(dst, seg, src, d);
+  return hipGetLastError();
+}
+
+hipError_t kafka_hy_add_ln(int f32, float* x, int64_t xs, const void* y, int64_t ys, const void* w, const void* b,
+                           float eps, int T, int d, void* out2, int64_t os, const void* w2, const void* b2,
+                           hipStream_t st) {
+  if (T <= 0) return hipSuccess;
+  const int mode = out2 == nullptr ? 0 : (w2 != nullptr ? 1 : 2);
+  DISPATCH_AT(f32, {
+    auto a = [&](auto k) {
+      k<<<T, NT, 0, st>>>(x, xs, (const AT*)y, ys, (const AT*)w, (const AT*)b, eps, d, (AT*)out2, os, (const AT*)w2,
+                          (const AT*)b2);
+    };
+    if (mode == 0) a(add_ln_kernel<AT, 0>);
+    else if (mode == 1) a(add_ln_kernel<AT, 1>);
+    else a(add_ln_kernel<AT, 2>);
+  });
+  return hipGetLastError();
+}
+
+hipError_t kafka_hy_gelu_mul(int f32, const void* gu, int64_t gs, void* out, int64_t T, int F, hipStream_t st) {
+  if (T * F <= 0) return hipSuccess;
+  DISPATCH_AT(f32, gelu_mul_kernel<AT><<<ew_grid(T * F), 256, 0, st>>>((const AT*)gu, gs, (AT*)out, T, F));
+  return hipGetLastError();
+}
+
+hipError_t kafka_hy_side_gate(int f32, const void* sg, int64_t ss, const int64_t* tokens, const void* emb, int64_t es,
+                              int col0, void* out, int64_t T, int dim, hipStream_t st) {
+  if (T * dim <= 0) return hipSuccess;
+  DISPATCH_AT(f32, side_gate_kernel<AT><<<ew_grid(T * dim), 256, 0, st>>>((const AT*)sg, ss, tokens, (const AT*)emb,
+                                                                          es, col0, (AT*)out, T, dim));
+  return hipGetLastError();
+}
+
+hipError_t kafka_hy_side_dwa(int f32, float* x, const void* y, int64_t ys, const void* sw, float eps, float* stack,
+                             int layer, const float* dwa, int64_t T, int d, hipStream_t st) {
+  if (T <= 0) return hipSuccess;
+  DISPATCH_AT(f32, side_dwa_kernel<AT><<<(int)T, NT, 0, st>>>(x, (const AT*)y, ys, (const AT*)sw, eps, stack, layer,
+                                                              dwa, T, d));
+  return hipGetLastError();
+}
+
+hipError_t kafka_hy_latent_prep(int f32, const void* qgd, int64_t qs, int T, int H, int dim, int rd, int R, int dkv_off,
+                                const void* dkv_w, float eps, const int64_t* positions, const float* cos_sin, int dims,
+                                void* cache, const int64_t* slots, void* q_rot, hipStream_t st) {
+  if (T <= 0) return hipSuccess;
+  DISPATCH_AT(f32, latent_prep_kernel<AT><<<T, NT, 0, st>>>((const AT*)qgd, qs, H, dim, rd, R, dkv_off,
+                                                           (const AT*)dkv_w, eps, positions, cos_sin, dims, (AT*)cache,
+                                                           slots, (AT*)q_rot));
+  return hipGetLastError();
+}
+
+hipError_t kafka_hy_sigmoid_mul(int f32, const void* a, int64_t a_h, int64_t a_t, const void* g, int64_t gs, void* out,
+                                int64_t T, int H, int vd, hipStream_t st) {
+  if (T * H * vd <= 0) return hipSuccess;
+  DISPATCH_AT(f32, sigmoid_mul_kernel<AT><<<ew_grid(T * H * vd), 256, 0, st>>>((const AT*)a, a_h, a_t, (const AT*)g,
+                                                                                gs, (AT*)out, T, H, vd));
+  return hipGetLastError();
+}
+
+// largest key-row length (latent + rotary part) the attention kernel holds in registers
+int kafka_hy_latent_attn_max_dk() { return 640; }
+
+hipError_t kafka_hy_latent_attn(int f32, const void* q_lat, int64_t ql_h, int64_t ql_t, const void* q_rot, int64_t qr_t,
+                                int64_t qr_h, const void* cache, int page, int R, int rd, const int* bt, int bt_stride,
+                                const int* tok_seg, const int64_t* positions, float scale, void* out, int64_t o_h,
+                                int64_t o_t, int T, int H, hipStream_t st) {
+  if (T <= 0) return hipSuccess;
+  constexpr int RPW = 4;
+  const int n_hg = (H + RPW - 1) / RPW;
+  const int64_t tasks = (int64_t)T * n_hg;
+  const int grid = (int)((tasks + 3) / 4);
+  const float sl = scale * 1.4426950408889634f;
+  const int Dk = R + rd;
+  DISPATCH_AT(f32, {
+    auto a = [&](auto k) {
+      k<<<grid, 256, 0, st>>>((const AT*)q_lat, ql_h, ql_t, (const AT*)q_rot, qr_t, qr_h, (const AT*)cache, page, R, rd,
+                              bt, bt_stride, tok_seg, positions, sl, (AT*)out, o_h, o_t, T, H, n_hg);
+    };
+    if (Dk <= 192) a(latent_attn_kernel<AT, 3, RPW, 4>);
+    else if (Dk <= 384) a(latent_attn_kernel<AT, 6, RPW, 4>);
+    else if (Dk <= 640) a(latent_attn_kernel<AT, 10, RPW, 2>);
+    else return hipErrorInvalidValue;
+  });
+  return hipGetLastError();
+}
+
+hipError_t kafka_hy_conv_silu(int f32, const void* proj, int64_t ps, int c0, const void* w, const void* b, int C,
+                              int taps, const int* tok_seg, const int* seg, int R, void* state, void* out, int64_t T,
+                              hipStream_t st) {
+  if (T <= 0 || taps > 8) return taps > 8 ? hipErrorInvalidValue : hipSuccess;
+  DISPATCH_AT(f32, {
+    conv_silu_kernel<AT><<<ew_grid(T * C), 256, 0, st>>>((const AT*)proj, ps, c0, (const AT*)w, (const AT*)b, C, taps,
+                                                         tok_seg, seg, (const AT*)state, (AT*)out, T);
+    if (taps > 1)
+      conv_state_kernel<AT><<<(int)(((int64_t)R * C + 255) / 256), 256, 0, st>>>((const AT*)proj, ps, c0, C, taps, seg,
+                                                                                (AT*)state, R);
+  });
+  return hipGetLastError();
+}
+
+// threads per workgroup = P * NG; 0 when the state does not fit the kernel's register budget
+int kafka_hy_scan_groups(int P, int N) {
+  if (P < 1 || P > 1024 || N < 1) return 0;
+  int ng = std::max(1, 256 / P);
+  if ((N + ng - 1) / ng > 32) ng = (N + 31) / 32;
+  return P * ng <= 1024 ? ng : 0;
+}
+
+hipError_t kafka_hy_ssm_scan(int f32, const void* xbc, int64_t xs, const void* proj, int64_t ps, int dt_off,
+                             const float* dt_bias, const float* A_log, const float* Dp, int heads, int P, int N, int G,
+                             const int* seg, int R, float* state, float* y, int64_t ys, hipStream_t st) {
+  if (R <= 0) return hipSuccess;
+  const int NG = kafka_hy_scan_groups(P, N);
+  if (NG == 0) return hipErrorInvalidValue;
+  const int ept = (N + NG - 1) / NG;
+  const size_t lds = sizeof(float) * (size_t)(2 * SCAN_TB * N + SCAN_TB * P + 2 * SCAN_TB + SCAN_TB * NG * P);
+  if (lds > 64 * 1024) return hipErrorInvalidValue;
+  DISPATCH_AT(f32, {
+    auto a = [&](auto k) {
+      k<<<R * heads, P * NG, lds, st>>>((const AT*)xbc, xs, (const AT*)proj, ps, dt_off, dt_bias, A_log, Dp, heads, P,
+                                        N, G, NG, seg, state, y, ys);
+    };
+    if (ept <= 8) a(ssm_scan_kernel<AT, 8>);
+    else if (ept <= 16) a(ssm_scan_kernel<AT, 16>);
+    else a(ssm_scan_kernel<AT, 32>);
+  });
+  return hipGetLastError();
+}
+
+hipError_t kafka_hy_gated_norm(int f32, const float* y, int64_t ys, const void* z, int64_t zs, const void* w, int inner,
+                               int groups, float eps, void* out, int64_t os, int64_t T, hipStream_t st) {
+  if (T <= 0) return hipSuccess;
+  DISPATCH_AT(f32, gated_norm_kernel<AT><<<dim3((unsigned)T, (unsigned)groups), NT, 0, st>>>(
+                       y, ys, (const AT*)z, zs, (const AT*)w, inner / groups, eps, (AT*)out, os));
+  return hipGetLastError();
+}
+
+}  // extern "C"

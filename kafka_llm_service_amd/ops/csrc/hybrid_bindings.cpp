@@ -1,0 +1,324 @@
+// Python bindings of the hybrid-family kernels (hybrid.hip). Shapes, dtypes, strides and index ranges that the
+// kernels assume are checked here, so a malformed call raises instead of launching.
+#include <torch/extension.h>
+#include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime.h>
+
+extern "C" {
+hipError_t kafka_hy_ln_shift(int f32, const float* x, int64_t xs, const void* w, const void* b, float eps, void* out,
+                             int64_t os, int T, int d, const void* mu, const int* tok_seg, const int* seg,
+                             const float* state, float* last, hipStream_t st);
+hipError_t kafka_hy_scatter_rows(float* dst, const int* seg, const float* src, int R, int d, hipStream_t st);
+hipError_t kafka_hy_add_ln(int f32, float* x, int64_t xs, const void* y, int64_t ys, const void* w, const void* b,
+                           float eps, int T, int d, void* out2, int64_t os, const void* w2, const void* b2,
+                           hipStream_t st);
+hipError_t kafka_hy_gelu_mul(int f32, const void* gu, int64_t gs, void* out, int64_t T, int F, hipStream_t st);
+hipError_t kafka_hy_side_gate(int f32, const void* sg, int64_t ss, const int64_t* tokens, const void* emb, int64_t es,
+                              int col0, void* out, int64_t T, int dim, hipStream_t st);
+hipError_t kafka_hy_side_dwa(int f32, float* x, const void* y, int64_t ys, const void* sw, float eps, float* stack,
+                             int layer, const float* dwa, int64_t T, int d, hipStream_t st);
+hipError_t kafka_hy_latent_prep(int f32, const void* qgd, int64_t qs, int T, int H, int dim, int rd, int R, int dkv_off,
+                                const void* dkv_w, float eps, const int64_t* positions, const float* cos_sin, int dims,
+                                void* cache, const int64_t* slots, void* q_rot, hipStream_t st);
+hipError_t kafka_hy_sigmoid_mul(int f32, const void* a, int64_t a_h, int64_t a_t, const void* g, int64_t gs, void* out,
+                                int64_t T, int H, int vd, hipStream_t st);
+int kafka_hy_latent_attn_max_dk();
+hipError_t kafka_hy_latent_attn(int f32, const void* q_lat, int64_t ql_h, int64_t ql_t, const void* q_rot, int64_t qr_t,
+                                int64_t qr_h, const void* cache, int page, int R, int rd, const int* bt, int bt_stride,
+                                const int* tok_seg, const int64_t* positions, float scale, void* out, int64_t o_h,
+                                int64_t o_t, int T, int H, hipStream_t st);
+hipError_t kafka_hy_conv_silu(int f32, const void* proj, int64_t ps, int c0, const void* w, const void* b, int C,
+                              int taps, const int* tok_seg, const int* seg, int R, void* state, void* out, int64_t T,
+                              hipStream_t st);
+int kafka_hy_scan_groups(int P, int N);
+hipError_t kafka_hy_ssm_scan(int f32, const void* xbc, int64_t xs, const void* proj, int64_t ps, int dt_off,
+                             const float* dt_bias, const float* A_log, const float* Dp, int heads, int P, int N, int G,
+                             const int* seg, int R, float* state, float* y, int64_t ys, hipStream_t st);
+hipError_t kafka_hy_gated_norm(int f32, const float* y, int64_t ys, const void* z, int64_t zs, const void* w, int inner,
+                               int groups, float eps, void* out, int64_t os, int64_t T, hipStream_t st);
+}
+
+namespace {
+
+#define HY_HIP(e)                                                                     \
+  do {                                                                                \
+    hipError_t _e = (e);                                                              \
+    TORCH_CHECK(_e == hipSuccess, "HIP launch failed: ", hipGetErrorString(_e));      \
+  } while (0)
+
+hipStream_t stream() { return c10::hip::getCurrentHIPStream().stream(); }
+
+using OptT = c10::optional<at::Tensor>;
+
+// the activation dtype of a call: every AT tensor must agree
+int act_f32(const at::Tensor& t) {
+  TORCH_CHECK(t.scalar_type() == at::kFloat || t.scalar_type() == at::kBFloat16, "activations must be bf16 or fp32");
+  return t.scalar_type() == at::kFloat;
+}
+void same_act(int f32, std::initializer_list<const at::Tensor*> ts) {
+  for (auto t : ts) TORCH_CHECK(t->is_cuda() && act_f32(*t) == f32, "mixed activation dtypes / not a GPU tensor");
+}
+void rows2d(const at::Tensor& t, const char* name) {
+  TORCH_CHECK(t.is_cuda() && t.dim() == 2 && t.stride(1) == 1, name, ": 2-D GPU tensor with contiguous rows expected");
+}
+void vec(const at::Tensor& t, int64_t n, const char* name) {
+  TORCH_CHECK(t.is_cuda() && t.is_contiguous() && t.numel() == n, name, ": contiguous vector of ", n, " expected");
+}
+void segs(const at::Tensor& tok_seg, const at::Tensor& seg, int64_t T) {
+  TORCH_CHECK(tok_seg.is_cuda() && tok_seg.scalar_type() == at::kInt && tok_seg.is_contiguous() &&
+                  tok_seg.numel() == T, "tok_seg: int32 [T]");
+  TORCH_CHECK(seg.is_cuda() && seg.scalar_type() == at::kInt && seg.is_contiguous() && seg.dim() == 2 &&
+                  seg.size(1) == 4, "seg: int32 [R, 4]");
+}
+
+void ln_shift(at::Tensor x, at::Tensor w, at::Tensor b, double eps, at::Tensor out, OptT mu, OptT tok_seg, OptT seg,
+              OptT state, OptT last) {
+  rows2d(x, "x"); rows2d(out, "out");
+  TORCH_CHECK(x.scalar_type() == at::kFloat, "ln_shift: x is the fp32 stream");
+  const int f32 = act_f32(out);
+  const int64_t T = x.size(0), d = x.size(1);
+  same_act(f32, {&w, &b});
+  vec(w, d, "w"); vec(b, d, "b");
+  TORCH_CHECK(out.size(0) == T && out.size(1) == d, "ln_shift: out shape");
+  const void* mup = nullptr; const int *tsp = nullptr, *sgp = nullptr; const float* stp = nullptr; float* lp = nullptr;
+  if (mu.has_value()) {
+    TORCH_CHECK(tok_seg.has_value() && seg.has_value() && state.has_value() && last.has_value(),
+                "ln_shift: a shift needs tok_seg, seg, state and last");
+    same_act(f32, {&*mu}); vec(*mu, d, "mu");
+    segs(*tok_seg, *seg, T);
+    TORCH_CHECK(state->is_cuda() && state->scalar_type() == at::kFloat && state->is_contiguous() && state->dim() == 2 &&
+                    state->size(1) == d, "ln_shift: state fp32 [slots, d]");
+    TORCH_CHECK(last->is_cuda() && last->scalar_type() == at::kFloat && last->is_contiguous() && last->dim() == 2 &&
+                    last->size(0) >= seg->size(0) && last->size(1) == d, "ln_shift: last fp32 [R, d]");
+    TORCH_CHECK(x.stride(0) >= d, "ln_shift: rows must not overlap");
+    mup = mu->data_ptr(); tsp = tok_seg->data_ptr<int>(); sgp = seg->data_ptr<int>();
+    stp = state->data_ptr<float>(); lp = last->data_ptr<float>();
+  }
+  HY_HIP(kafka_hy_ln_shift(f32, x.data_ptr<float>(), x.stride(0), w.data_ptr(), b.data_ptr(), (float)eps,
+                           out.data_ptr(), out.stride(0), (int)T, (int)d, mup, tsp, sgp, stp, lp, stream()));
+}
+
+void scatter_rows(at::Tensor dst, at::Tensor seg, at::Tensor src) {
+  TORCH_CHECK(dst.is_cuda() && dst.scalar_type() == at::kFloat && dst.is_contiguous() && dst.dim() == 2 &&
+                  src.is_cuda() && src.scalar_type() == at::kFloat && src.is_contiguous() && src.dim() == 2 &&
+                  src.size(1) == dst.size(1) && seg.is_cuda() && seg.scalar_type() == at::kInt &&
+                  seg.is_contiguous() && seg.dim() == 2 && seg.size(1) == 4 && src.size(0) >= seg.size(0),
+              "scatter_rows: fp32 [slots, d] <- fp32 [R, d] by int32 seg [R, 4]");
+  HY_HIP(kafka_hy_scatter_rows(dst.data_ptr<float>(), seg.data_ptr<int>(), src.data_ptr<float>(), (int)seg.size(0),
+                               (int)dst.size(1), stream()));
+}
+
+void add_ln(at::Tensor x, at::Tensor y, at::Tensor w, at::Tensor b, double eps, OptT out2, OptT w2, OptT b2) {
+  rows2d(x, "x"); rows2d(y, "y");
+  TORCH_CHECK(x.scalar_type() == at::kFloat, "add_ln: x is the fp32 stream");
+  const int f32 = act_f32(y);
+  const int64_t T = x.size(0), d = x.size(1);
+  same_act(f32, {&w, &b});
+  vec(w, d, "w"); vec(b, d, "b");
+  TORCH_CHECK(y.size(0) == T && y.size(1) == d && x.stride(0) >= d, "add_ln: shapes");
+  void* o2 = nullptr; int64_t os = 0; const void *w2p = nullptr, *b2p = nullptr;
+  if (out2.has_value()) {
+    rows2d(*out2, "out2"); same_act(f32, {&*out2});
+    TORCH_CHECK(out2->size(0) == T && out2->size(1) == d, "add_ln: out2 shape");
+    o2 = out2->data_ptr(); os = out2->stride(0);
+    if (w2.has_value()) {
+      TORCH_CHECK(b2.has_value(), "add_ln: w2 without b2");
+      same_act(f32, {&*w2, &*b2}); vec(*w2, d, "w2"); vec(*b2, d, "b2");
+      w2p = w2->data_ptr(); b2p = b2->data_ptr();
+    }
+  }
+  HY_HIP(kafka_hy_add_ln(f32, x.data_ptr<float>(), x.stride(0), y.data_ptr(), y.stride(0), w.data_ptr(), b.data_ptr(),
+                         (float)eps, (int)T, (int)d, o2, os, w2p, b2p, stream()));
+}
+
+void gelu_mul(at::Tensor gu, at::Tensor out) {
+  rows2d(gu, "gu");
+  const int f32 = act_f32(gu);
+  same_act(f32, {&out});
+  TORCH_CHECK(out.is_contiguous() && out.dim() == 2 && out.size(0) == gu.size(0) && gu.size(1) == 2 * out.size(1),
+              "gelu_mul: [T, 2F] -> [T, F]");
+  HY_HIP(kafka_hy_gelu_mul(f32, gu.data_ptr(), gu.stride(0), out.data_ptr(), gu.size(0), (int)out.size(1), stream()));
+}
+
+void side_gate(at::Tensor sg, at::Tensor tokens, at::Tensor emb, int64_t col0, at::Tensor out) {
+  rows2d(sg, "sg"); rows2d(emb, "emb");
+  const int f32 = act_f32(sg);
+  same_act(f32, {&emb, &out});
+  const int64_t T = sg.size(0), dim = sg.size(1);
+  TORCH_CHECK(tokens.is_cuda() && tokens.scalar_type() == at::kLong && tokens.is_contiguous() && tokens.numel() == T,
+              "side_gate: tokens int64 [T]");
+  TORCH_CHECK(out.is_contiguous() && out.dim() == 2 && out.size(0) == T && out.size(1) == dim && col0 >= 0 &&
+                  col0 + dim <= emb.size(1), "side_gate: shapes");
+  HY_HIP(kafka_hy_side_gate(f32, sg.data_ptr(), sg.stride(0), tokens.data_ptr<int64_t>(), emb.data_ptr(),
+                            emb.stride(0), (int)col0, out.data_ptr(), T, (int)dim, stream()));
+}
+
+void side_dwa(at::Tensor x, OptT y, OptT sw, double eps, OptT stack, int64_t layer, OptT dwa) {
+  TORCH_CHECK(x.is_cuda() && x.scalar_type() == at::kFloat && x.is_contiguous() && x.dim() == 2,
+              "side_dwa: x fp32 [T, d] contiguous");
+  const int64_t T = x.size(0), d = x.size(1);
+  int f32 = 0; const void *yp = nullptr, *swp = nullptr; int64_t ys = 0;
+  if (y.has_value()) {
+    TORCH_CHECK(sw.has_value(), "side_dwa: y without its norm weight");
+    rows2d(*y, "y");
+    f32 = act_f32(*y);
+    same_act(f32, {&*sw}); vec(*sw, d, "side weight");
+    TORCH_CHECK(y->size(0) == T && y->size(1) == d, "side_dwa: y shape");
+    yp = y->data_ptr(); swp = sw->data_ptr(); ys = y->stride(0);
+  }
+  float* sp = nullptr; const float* dp = nullptr;
+  if (stack.has_value()) {
+    TORCH_CHECK(stack->is_cuda() && stack->scalar_type() == at::kFloat && stack->is_contiguous() && stack->dim() == 3 &&
+                    stack->size(1) == T && stack->size(2) == d && layer >= 0 && layer + 1 < stack->size(0),
+                "side_dwa: stack fp32 [layers + 1, T, d]");
+    sp = stack->data_ptr<float>();
+    if (dwa.has_value()) {
+      TORCH_CHECK(dwa->is_cuda() && dwa->scalar_type() == at::kFloat && dwa->is_contiguous() &&
+                      dwa->numel() == layer + 2, "side_dwa: dwa fp32 [layer + 2]");
+      dp = dwa->data_ptr<float>();
+    }
+  }
+  HY_HIP(kafka_hy_side_dwa(f32, x.data_ptr<float>(), yp, ys, swp, (float)eps, sp, (int)layer, dp, T, (int)d, stream()));
+}
+
+void latent_prep(at::Tensor qgd, int64_t H, int64_t dim, int64_t rd, int64_t R, int64_t dkv_off, OptT dkv_w, double eps,
+                 at::Tensor positions, at::Tensor cos_sin, int64_t dims, at::Tensor cache, at::Tensor slots,
+                 at::Tensor q_rot) {
+  rows2d(qgd, "qgd");
+  const int f32 = act_f32(qgd);
+  same_act(f32, {&cache, &q_rot});
+  const int64_t T = qgd.size(0);
+  TORCH_CHECK(H > 0 && dim >= 0 && rd > 0 && R > 0 && dims > 0 && dims % 2 == 0 && dims <= rd &&
+                  H * (dim + rd) <= qgd.size(1), "latent_prep: head sizes");
+  TORCH_CHECK(positions.is_cuda() && positions.scalar_type() == at::kLong && positions.is_contiguous() &&
+                  positions.numel() == T && slots.is_cuda() && slots.scalar_type() == at::kLong &&
+                  slots.is_contiguous() && slots.numel() == T, "latent_prep: positions / slots int64 [T]");
+  TORCH_CHECK(cos_sin.is_cuda() && cos_sin.scalar_type() == at::kFloat && cos_sin.is_contiguous() &&
+                  cos_sin.dim() == 2 && cos_sin.size(1) == dims, "latent_prep: cos_sin fp32 [positions, dims]");
+  TORCH_CHECK(q_rot.is_contiguous() && q_rot.dim() == 3 && q_rot.size(0) == T && q_rot.size(1) == H &&
+                  q_rot.size(2) == rd, "latent_prep: q_rot [T, H, rot_dim]");
+  TORCH_CHECK(cache.is_contiguous() && cache.dim() == 3 && cache.size(2) == R + rd, "latent_prep: cache [pages, page, "
+              "kv_rank + rot_dim]");
+  const void* wp = nullptr;
+  if (dkv_off >= 0) {
+    TORCH_CHECK(dkv_w.has_value() && dkv_off + R + rd <= qgd.size(1), "latent_prep: latent columns");
+    same_act(f32, {&*dkv_w}); vec(*dkv_w, R, "latent norm weight");
+    wp = dkv_w->data_ptr();
+  }
+  HY_HIP(kafka_hy_latent_prep(f32, qgd.data_ptr(), qgd.stride(0), (int)T, (int)H, (int)dim, (int)rd, (int)R,
+                              (int)dkv_off, wp, (float)eps, positions.data_ptr<int64_t>(), cos_sin.data_ptr<float>(),
+                              (int)dims, cache.data_ptr(), slots.data_ptr<int64_t>(), q_rot.data_ptr(), stream()));
+}
+
+void sigmoid_mul(at::Tensor a, at::Tensor g, at::Tensor out) {
+  const int f32 = act_f32(a);
+  same_act(f32, {&g, &out});
+  rows2d(g, "g");
+  TORCH_CHECK(a.dim() == 3 && a.stride(2) == 1, "sigmoid_mul: a [H, T, v]");
+  const int64_t H = a.size(0), T = a.size(1), vd = a.size(2);
+  TORCH_CHECK(g.size(0) == T && g.size(1) == H * vd && out.is_contiguous() && out.dim() == 2 && out.size(0) == T &&
+                  out.size(1) == H * vd, "sigmoid_mul: shapes");
+  HY_HIP(kafka_hy_sigmoid_mul(f32, a.data_ptr(), a.stride(0), a.stride(1), g.data_ptr(), g.stride(0), out.data_ptr(), T,
+                              (int)H, (int)vd, stream()));
+}
+
+void latent_attn(at::Tensor q_lat, at::Tensor q_rot, at::Tensor cache, at::Tensor bt, at::Tensor tok_seg,
+                 at::Tensor positions, double scale, at::Tensor out) {
+  const int f32 = act_f32(q_lat);
+  same_act(f32, {&q_rot, &cache, &out});
+  TORCH_CHECK(q_lat.dim() == 3 && q_lat.stride(2) == 1 && out.dim() == 3 && out.stride(2) == 1 && q_rot.dim() == 3 &&
+                  q_rot.stride(2) == 1, "latent_attn: q_lat / out [H, T, R], q_rot [T, H, rot_dim]");
+  const int64_t H = q_lat.size(0), T = q_lat.size(1), R = q_lat.size(2), rd = q_rot.size(2);
+  TORCH_CHECK(q_rot.size(0) == T && q_rot.size(1) == H && out.size(0) == H && out.size(1) == T && out.size(2) == R,
+              "latent_attn: shapes");
+  TORCH_CHECK(cache.is_contiguous() && cache.dim() == 3 && cache.size(2) == R + rd, "latent_attn: cache row");
+  TORCH_CHECK(R + rd <= kafka_hy_latent_attn_max_dk(), "latent_attn: kv_rank + rot_dim beyond ",
+              kafka_hy_latent_attn_max_dk());
+  TORCH_CHECK(bt.is_cuda() && bt.scalar_type() == at::kInt && bt.dim() == 2 && bt.stride(1) == 1 &&
+                  tok_seg.is_cuda() && tok_seg.scalar_type() == at::kInt && tok_seg.is_contiguous() &&
+                  tok_seg.numel() == T && positions.is_cuda() && positions.scalar_type() == at::kLong &&
+                  positions.is_contiguous() && positions.numel() == T, "latent_attn: block tables / tok_seg / positions");
+  HY_HIP(kafka_hy_latent_attn(f32, q_lat.data_ptr(), q_lat.stride(0), q_lat.stride(1), q_rot.data_ptr(),
+                              q_rot.stride(0), q_rot.stride(1), cache.data_ptr(), (int)cache.size(1), (int)R, (int)rd,
+                              bt.data_ptr<int>(), (int)bt.stride(0), tok_seg.data_ptr<int>(),
+                              positions.data_ptr<int64_t>(), (float)scale, out.data_ptr(), out.stride(0), out.stride(1),
+                              (int)T, (int)H, stream()));
+}
+
+void conv_silu(at::Tensor proj, int64_t c0, at::Tensor w, at::Tensor b, at::Tensor tok_seg, at::Tensor seg,
+               at::Tensor state, at::Tensor out) {
+  rows2d(proj, "proj");
+  const int f32 = act_f32(proj);
+  same_act(f32, {&w, &b, &state, &out});
+  const int64_t T = proj.size(0);
+  TORCH_CHECK(w.is_contiguous() && w.dim() == 2, "conv_silu: w [C, taps]");
+  const int64_t C = w.size(0), taps = w.size(1);
+  vec(b, C, "conv bias");
+  segs(tok_seg, seg, T);
+  TORCH_CHECK(taps >= 1 && taps <= 8 && c0 >= 0 && c0 + C <= proj.size(1) && out.is_contiguous() && out.dim() == 2 &&
+                  out.size(0) == T && out.size(1) == C, "conv_silu: shapes");
+  TORCH_CHECK(state.is_contiguous() && state.dim() == 3 && state.size(1) == taps - 1 && state.size(2) == C,
+              "conv_silu: state [slots, taps - 1, C]");
+  HY_HIP(kafka_hy_conv_silu(f32, proj.data_ptr(), proj.stride(0), (int)c0, w.data_ptr(), b.data_ptr(), (int)C,
+                            (int)taps, tok_seg.data_ptr<int>(), seg.data_ptr<int>(), (int)seg.size(0),
+                            state.data_ptr(), out.data_ptr(), T, stream()));
+}
+
+void ssm_scan(at::Tensor xbc, at::Tensor proj, int64_t dt_off, at::Tensor dt_bias, at::Tensor A_log, at::Tensor D,
+              int64_t heads, int64_t P, int64_t N, int64_t G, at::Tensor seg, at::Tensor state, at::Tensor y) {
+  rows2d(xbc, "xbc"); rows2d(proj, "proj"); rows2d(y, "y");
+  const int f32 = act_f32(xbc);
+  same_act(f32, {&proj});
+  const int64_t T = xbc.size(0);
+  TORCH_CHECK(heads > 0 && G > 0 && heads % G == 0 && xbc.size(1) == heads * P + 2 * G * N && proj.size(0) == T &&
+                  dt_off >= 0 && dt_off + heads <= proj.size(1), "ssm_scan: sizes");
+  for (const at::Tensor* t : {&dt_bias, &A_log, &D})
+    TORCH_CHECK(t->is_cuda() && t->scalar_type() == at::kFloat && t->is_contiguous() && t->numel() == heads,
+                "ssm_scan: dt_bias / A_log / D fp32 [heads]");
+  TORCH_CHECK(seg.is_cuda() && seg.scalar_type() == at::kInt && seg.is_contiguous() && seg.dim() == 2 &&
+                  seg.size(1) == 4, "ssm_scan: seg int32 [R, 4]");
+  TORCH_CHECK(state.is_cuda() && state.scalar_type() == at::kFloat && state.is_contiguous() && state.dim() == 4 &&
+                  state.size(1) == heads && state.size(2) == N && state.size(3) == P,
+              "ssm_scan: state fp32 [slots, heads, N, P]");
+  TORCH_CHECK(y.scalar_type() == at::kFloat && y.size(0) == T && y.size(1) == heads * P, "ssm_scan: y fp32 [T, inner]");
+  TORCH_CHECK(kafka_hy_scan_groups((int)P, (int)N) > 0, "ssm_scan: state of ", N, " x ", P, " per head is not supported");
+  HY_HIP(kafka_hy_ssm_scan(f32, xbc.data_ptr(), xbc.stride(0), proj.data_ptr(), proj.stride(0), (int)dt_off,
+                           dt_bias.data_ptr<float>(), A_log.data_ptr<float>(), D.data_ptr<float>(), (int)heads, (int)P,
+                           (int)N, (int)G, seg.data_ptr<int>(), (int)seg.size(0), state.data_ptr<float>(),
+                           y.data_ptr<float>(), y.stride(0), stream()));
+}
+
+void gated_norm(at::Tensor y, at::Tensor proj, at::Tensor w, int64_t groups, double eps, at::Tensor out) {
+  rows2d(y, "y"); rows2d(proj, "proj"); rows2d(out, "out");
+  const int f32 = act_f32(proj);
+  same_act(f32, {&w, &out});
+  const int64_t T = y.size(0), inner = y.size(1);
+  TORCH_CHECK(y.scalar_type() == at::kFloat && proj.size(0) == T && proj.size(1) >= inner && groups > 0 &&
+                  groups < 65536 && inner % groups == 0 && out.size(0) == T && out.size(1) == inner,
+              "gated_norm: shapes");
+  vec(w, inner, "norm weight");
+  HY_HIP(kafka_hy_gated_norm(f32, y.data_ptr<float>(), y.stride(0), proj.data_ptr(), proj.stride(0), w.data_ptr(),
+                             (int)inner, (int)groups, (float)eps, out.data_ptr(), out.stride(0), T, stream()));
+}
+
+}  // namespace
+
+void kafka_bind_hybrid(pybind11::module_& m) {
+  namespace py = pybind11;
+  m.def("hy_ln_shift", &ln_shift, py::arg("x"), py::arg("w"), py::arg("b"), py::arg("eps"), py::arg("out"),
+        py::arg("mu") = py::none(), py::arg("tok_seg") = py::none(), py::arg("seg") = py::none(),
+        py::arg("state") = py::none(), py::arg("last") = py::none());
+  m.def("hy_scatter_rows", &scatter_rows);
+  m.def("hy_add_ln", &add_ln, py::arg("x"), py::arg("y"), py::arg("w"), py::arg("b"), py::arg("eps"),
+        py::arg("out2") = py::none(), py::arg("w2") = py::none(), py::arg("b2") = py::none());
+  m.def("hy_gelu_mul", &gelu_mul);
+  m.def("hy_side_gate", &side_gate);
+  m.def("hy_side_dwa", &side_dwa);
+  m.def("hy_latent_prep", &latent_prep);
+  m.def("hy_sigmoid_mul", &sigmoid_mul);
+  m.def("hy_latent_attn", &latent_attn);
+  m.def("hy_conv_silu", &conv_silu);
+  m.def("hy_ssm_scan", &ssm_scan);
+  m.def("hy_gated_norm", &gated_norm);
+  m.def("hy_scan_groups", [](int P, int N) { return kafka_hy_scan_groups(P, N); });
+}

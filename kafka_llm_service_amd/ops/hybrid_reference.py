@@ -38,7 +38,7 @@ def ln_shift(x, w, b, eps, out, mu=None, tok_seg=None, seg=None, state=None, las
 
 
 def scatter_rows(dst, seg, src):
-    dst[seg[:, 3].long()] = src.to(dst.dtype)
+    dst[seg[:, 3].long()] = src[:seg.shape[0]].to(dst.dtype)
 
 
 def add_ln(x, y, w, b, eps, out2=None, w2=None, b2=None):
