@@ -277,7 +277,12 @@ class BuduraxLM:
 
         self.embed = f32("embed")  # the residual stream starts (and stays) fp32; bf16 values are exact in it
         self.side_embed = act("side.embed") if cfg.token_side_dim else None
-        self.final_norm, self.final_norm_b, self.head = act("final.norm"), act("final.norm.b"), act("head")
+        self.final_norm, self.final_norm_b = act("final.norm"), act("final.norm.b")
+        # the sampler reads logits rows in 8-element vectors: the head is padded with zero rows to a multiple of 8
+        # and the extra columns are cut off as a view
+        pad = -cfg.vocab_size % 8
+        self.head = torch.cat([W["head"].to(dt), torch.zeros(pad, cfg.hidden_size, dtype=dt)], 0).to(dev).contiguous()
+        self._tensors.append(self.head)
         self.layers = []
         for i, L in enumerate(cfg.layers):
             p, m = f"l{i}.", L["mixer"]
@@ -418,7 +423,7 @@ class BuduraxLM:
         xs = x.index_select(0, inp.logit_rows)
         hf = torch.empty(xs.shape[0], d, dtype=dt, device=dev)
         hops.ln_shift(xs, self.final_norm, self.final_norm_b, eps, hf)
-        return F.linear(hf, self.head).float()
+        return F.linear(hf, self.head).float()[:, :cfg.vocab_size]
 
     def _latent_attention(self, i: int, lw, h, inp, m: SegMeta, pages: list) -> torch.Tensor:
         mm = lw.m

@@ -16,7 +16,7 @@ from kafka_llm_service_amd.engine.sequence import SamplingParams
 from kafka_llm_service_amd.models import budurax as bx
 from kafka_llm_service_amd.ops import hybrid as hops
 
-DEVICES = ["cpu", pytest.param("cuda", marks=pytest.mark.gpu)]
+DEVICES = ["cpu", pytest.param("cuda:0", marks=pytest.mark.gpu)]
 
 
 def _attn(heads=3, dim=24, rot_dim=16, dims=8, vdim=20, rank=40, scaling=True, kv_from=None, scale=None):
