@@ -94,7 +94,93 @@ def parse(argv=None):
                     help="paged KV cache precision (fp8 = e4m3 + per-token scales; an opt-in A/B, not the headline)")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--json-out", default=None)
+    ap.add_argument("--arch-compare", action="store_true",
+                    help="instead of the headline workload: prefill and decode tok/s of a Budurax model (latent "
+                         "attention + Mamba-2 layers) beside a Llama model of the same width, heads, depth, "
+                         "feed-forward and vocabulary (random weights), one JSON line per measurement")
+    ap.add_argument("--arch-width", type=int, default=4096)
+    ap.add_argument("--arch-layers", type=int, default=6)
+    ap.add_argument("--arch-prefill", default="512,2048,8192", help="prompt lengths of the prefill measurements")
+    ap.add_argument("--arch-decode", default="16x2048,64x2048,64x8192",
+                    help="decode measurements as <sequences>x<context tokens>")
+    ap.add_argument("--arch-models", default="budurax,llama")
     return ap.parse_args(argv)
+
+
+def arch_compare(args) -> int:
+    """Prefill and decode throughput of the two model families at equal layer sizes, each through its own engine
+    (LLMEngine.feed: explicit steps, no sampling): a whole prompt of S tokens as one step, and single-token steps of
+    B sequences at a context of C tokens. Times are HIP-event times of the steps alone."""
+    import torch
+
+    from kafka_llm_service_amd.engine.engine import EngineConfig, LLMEngine
+    from kafka_llm_service_amd.models.config import ModelConfig, _budurax
+    from kafka_llm_service_amd.models.budurax import BuduraxConfig
+
+    dev = "cuda:0" if torch.cuda.is_available() else "cpu"
+    w, L = args.arch_width, args.arch_layers
+    heads, ff, vocab = w // 128, int(w * 3.5), 32000
+    prefills = [int(x) for x in args.arch_prefill.split(",") if x]
+    decodes = [tuple(int(v) for v in x.split("x")) for x in args.arch_decode.split(",") if x]
+    need = max([max(prefills, default=0)] + [b * (c + 64) for b, c in decodes]) + 64
+    cfgs = {"budurax": BuduraxConfig.from_dict(_budurax(w, heads, L, vocab, ff), name=f"budurax-w{w}-l{L}"),
+            "llama": ModelConfig(name=f"llama-w{w}-l{L}", hidden_size=w, intermediate_size=ff, num_layers=L,
+                                 num_heads=heads, num_kv_heads=max(1, heads // 4), vocab_size=vocab,
+                                 max_position_embeddings=131072, bos_token_id=1, eos_token_ids=[2])}
+    rng = random.Random(args.seed)
+
+    def timed(fn) -> float:
+        if dev == "cpu":
+            t0 = time.perf_counter()
+            fn()
+            return (time.perf_counter() - t0) * 1e3
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b)
+
+    lines = []
+    for name in [m for m in args.arch_models.split(",") if m]:
+        mc = cfgs[name]
+        eng = LLMEngine(EngineConfig(model=mc.name, device=dev, seed=args.seed, num_kv_blocks=-(-need // 16) + 8,
+                                     max_num_seqs=max(b for b, _ in decodes) if decodes else 4,
+                                     max_model_len=max([max(prefills, default=0)] + [c + 128 for _, c in decodes]) + 64,
+                                     enable_prefix_cache=False, use_cascade=False, async_scheduling=False),
+                        model_cfg=mc)
+        base = {"model": mc.name, "params_b": round(mc.num_params() / 1e9, 3), "dtype": "bf16", "data": "synthetic"}
+        n = 0
+        for S in prefills:
+            ms = []
+            for _ in range(3):
+                n += 1
+                toks = [rng.randrange(vocab) for _ in range(S)]
+                ms.append(timed(lambda: eng.feed([(f"p{n}", toks, [S - 1])], [f"p{n}"])))
+            lines.append(dict(base, phase="prefill", tokens=S, ms=round(min(ms), 3),
+                              tok_s=round(S / min(ms) * 1e3, 1)))
+            print(json.dumps(lines[-1]), flush=True)
+        for B, C in decodes:
+            ids = [f"d{n}-{i}" for i in range(B)]
+            n += 1
+            for i in ids:  # contexts built one sequence a step
+                eng.feed([(i, [rng.randrange(vocab) for _ in range(C)], [])])
+            step = lambda: eng.feed([(i, [rng.randrange(vocab)], [0]) for i in ids])  # noqa: E731
+            for _ in range(max(1, args.warmup // 4)):
+                step()
+            k = max(4, min(args.steps, 32))
+            ms = sorted(timed(step) for _ in range(k))
+            eng.feed([], ids)
+            lines.append(dict(base, phase="decode", sequences=B, context=C, ms_per_step=round(ms[len(ms) // 2], 3),
+                              tok_s=round(B / ms[len(ms) // 2] * 1e3, 1)))
+            print(json.dumps(lines[-1]), flush=True)
+        del eng
+        if dev != "cpu":
+            torch.cuda.empty_cache()
+    if args.json_out:
+        with open(args.json_out, "w") as f:
+            json.dump(lines, f, indent=1)
+    return 0
 
 
 # ---------------------------------------------------------------------------------------------------------------
@@ -254,6 +340,8 @@ def stratified_budgets(threads, args, rng: random.Random) -> list[tuple[int, int
 
 def main(argv=None):
     args = parse(argv)
+    if args.arch_compare:
+        return arch_compare(args)
     if "WORLD_SIZE" not in os.environ and args.gpus > 1:
         return spawn_ranks(args.gpus)
     from kafka_llm_service_amd.utils.affinity import pin_local_process

@@ -61,6 +61,7 @@ class HostStep:
     # bt_w] | row -> run [T] | runs [n_seg, 4] = (first row, rows, first position, state slot)
     n_seg: int = 0
     owners: list = field(default_factory=list)  # with ``want``: (seq_id, offset) of every logit row, in row order
+    tiles: list = field(default_factory=list)   # segment plans: (tile tokens, first int32 word, tiles) per tile size
 
 
 @dataclass
@@ -595,7 +596,16 @@ class ModelRunner:
         h = HostStep(B=len(batch.decode), T=T, nbt=max(1, R), bt_w=bt_w, bt_need=min(need, bt_w),
                      n_rows=len(logit_rows), patch=patch, n_seg=R, owners=owners)
         h.i64 = np.concatenate([tokens, positions, slots, np.asarray(logit_rows, dtype=np.int64)])
-        h.i32 = np.concatenate([bt.reshape(-1), tok_seg, seg.reshape(-1)])
+        parts = [bt.reshape(-1), tok_seg, seg.reshape(-1)]
+        off = sum(p.size for p in parts)
+        for tt in getattr(self.model, "attn_tile_tokens", ()):
+            # attention tiles of at most tt tokens, none across two runs
+            it = np.asarray([(q0 + a, min(tt, n - a), j, 0) for j, (q0, n, _, _) in enumerate(seg[:R].tolist())
+                             for a in range(0, n, tt)], dtype=np.int32).reshape(-1, 4)
+            h.tiles.append((tt, off, it.shape[0]))
+            parts.append(it.reshape(-1))
+            off += it.size
+        h.i32 = np.concatenate(parts)
         h.stats = {"B": h.B, "T": T, "segments": R}
         return h, sample_seqs
 
@@ -843,7 +853,8 @@ class ModelRunner:
 
             n_bt = nbt * h.bt_w
             sm = SegMeta(T, h.n_seg, d32[n_bt + T:n_bt + T + 4 * h.n_seg].view(h.n_seg, 4), d32[n_bt:n_bt + T],
-                         d32[:n_bt].view(nbt, h.bt_w))
+                         d32[:n_bt].view(nbt, h.bt_w),
+                         {tt: d32[o:o + 4 * n].view(n, 4) for tt, o, n in h.tiles})
             if h.n_late:
                 L, n = h.late_off, h.n_late
                 t_tokens.index_copy_(0, d64[L:L + n], self.tok_buf.index_select(0, d64[L + n:L + 2 * n]))

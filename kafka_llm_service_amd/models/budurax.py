@@ -132,36 +132,46 @@ def tensor_shapes(cfg: BuduraxConfig, shift: bool = True, dwa: bool = True) -> d
     return s
 
 
-def random_tensors(cfg: BuduraxConfig, seed: int = 0, shift: bool = True, dwa: bool = True) -> dict[str, torch.Tensor]:
-    """Seeded bf16 weights with the value ranges each kind of tensor needs (decays in (0, 1), positive step sizes)."""
-    g = torch.Generator().manual_seed(seed)
+def random_tensors(cfg: BuduraxConfig, seed: int = 0, shift: bool = True, dwa: bool = True,
+                   device="cpu") -> dict[str, torch.Tensor]:
+    """Seeded bf16 weights with the value ranges each kind of tensor needs (decays in (0, 1), positive step sizes),
+    drawn on ``device`` (large models: on the GPU)."""
+    g = torch.Generator(device=device).manual_seed(seed)
+
+    def rn(shape):
+        return torch.randn(shape, generator=g, device=device)
+
+    def ru(shape):
+        return torch.rand(shape, generator=g, device=device)
+
+
     out = {}
     for name, shape in tensor_shapes(cfg, shift, dwa).items():
         leaf = name.split(".")[-1]
         if name.endswith(".b"):
-            t = 0.1 * torch.randn(shape, generator=g)
+            t = 0.1 * rn(shape)
         elif leaf in ("norm1", "norm2", "norm1b", "norm2b") or name in ("final.norm",) or name.endswith("side.norm") \
                 or name.endswith("dkv.norm") or name.endswith("mix.norm"):
-            t = 1.0 + 0.1 * torch.randn(shape, generator=g)
+            t = 1.0 + 0.1 * rn(shape)
             if leaf in ("norm1b", "norm2b") or name.endswith("side.norm"):
                 t = t * 0.5
         elif leaf == "shift":
-            t = torch.rand(shape, generator=g)
+            t = ru(shape)
         elif leaf == "dwa":
-            t = torch.rand(shape, generator=g) + 0.2
+            t = ru(shape) + 0.2
             t = t / t.sum()
         elif leaf == "A_log":
-            t = torch.log(1.0 + 7.0 * torch.rand(shape, generator=g))
+            t = torch.log(1.0 + 7.0 * ru(shape))
         elif leaf == "dt_bias":
-            t = torch.log(torch.expm1(0.01 + 0.2 * torch.rand(shape, generator=g)))
+            t = torch.log(torch.expm1(0.01 + 0.2 * ru(shape)))
         elif leaf == "D":
-            t = 1.0 + 0.1 * torch.randn(shape, generator=g)
+            t = 1.0 + 0.1 * rn(shape)
         elif leaf == "conv":
-            t = torch.randn(shape, generator=g) / math.sqrt(shape[1])
+            t = rn(shape) / math.sqrt(shape[1])
         elif leaf == "embed":
-            t = torch.randn(shape, generator=g)
+            t = rn(shape)
         else:
-            t = torch.randn(shape, generator=g) / math.sqrt(shape[-1])
+            t = rn(shape) / math.sqrt(shape[-1])
         out[name] = t.to(torch.bfloat16)
     return out
 
@@ -200,6 +210,8 @@ class SegMeta:
     seg: torch.Tensor
     tok_seg: torch.Tensor
     block_tables: torch.Tensor
+    # attention tiles per tile size in tokens: int32 [n, 4] = (first row, tokens, run, 0), each within one run
+    tiles: dict = field(default_factory=dict)
 
 
 @dataclass
@@ -271,7 +283,7 @@ class BuduraxLM:
             return t
 
         def fused(names):
-            t = torch.cat([W[n].to(dt) for n in names], 0).to(dev).contiguous()
+            t = torch.cat([W[n].to(device=dev, dtype=dt) for n in names], 0).contiguous()
             self._tensors.append(t)
             return t
 
@@ -281,7 +293,8 @@ class BuduraxLM:
         # the sampler reads logits rows in 8-element vectors: the head is padded with zero rows to a multiple of 8
         # and the extra columns are cut off as a view
         pad = -cfg.vocab_size % 8
-        self.head = torch.cat([W["head"].to(dt), torch.zeros(pad, cfg.hidden_size, dtype=dt)], 0).to(dev).contiguous()
+        hw = W["head"].to(device=dev, dtype=dt)
+        self.head = torch.cat([hw, torch.zeros(pad, cfg.hidden_size, dtype=dt, device=dev)], 0).contiguous()
         self._tensors.append(self.head)
         self.layers = []
         for i, L in enumerate(cfg.layers):
@@ -341,6 +354,9 @@ class BuduraxLM:
                 lw.side_gate = lw.side_proj = lw.side_norm = None
             self.layers.append(lw)
         self.has_dwa = any(lw.dwa is not None for lw in self.layers)
+        # tile sizes (tokens) the step plan must carry for the attention layers (ops.hybrid.tile_tokens)
+        self.attn_tile_tokens = sorted({hops.tile_tokens(int(lw.m["heads"])) for lw in self.layers
+                                        if lw.type == "latent_attention"})
         return self
 
     def _rot_table(self, rot: dict) -> torch.Tensor:
@@ -353,7 +369,9 @@ class BuduraxLM:
     def page_bytes(self) -> int:
         """Bytes of one 16-token page over every layer that owns a latent cache."""
         es = torch.empty(0, dtype=self.dtype).element_size()
-        return sum(PAGE * (int(L["mixer"]["kv_rank"]) + int(L["mixer"]["rot_dim"])) * es for L in self.cfg.layers
+        # (the latent part is kept twice where the matrix-core kernel runs: row-major and page-wise transposed)
+        return sum(PAGE * (2 * int(L["mixer"]["kv_rank"]) + int(L["mixer"]["rot_dim"])) * es
+                   for L in self.cfg.layers
                    if L["type"] == "latent_attention" and L["mixer"].get("kv_from") is None) or 1
 
     def alloc_cache(self, num_blocks: int, num_slots: int) -> tuple[list, RecurrentState]:
@@ -361,11 +379,15 @@ class BuduraxLM:
         a masked key's row is never read, but fresh memory must not hold NaN patterns for the debug checks."""
         dev, dt, d = self.device, self.dtype, self.cfg.hidden_size
         pages, shift, conv, ssm = [], [], [], []
+        self.pages_t = []  # page-wise transposed latent copies [blocks, kv_rank, 16] where the MFMA kernel applies
         for lw in self.layers:
             m = lw.m
             own = lw.type == "latent_attention" and lw.kv_from is None
             pages.append(torch.zeros(num_blocks, PAGE, int(m["kv_rank"]) + int(m["rot_dim"]), dtype=dt, device=dev)
                          if own else None)
+            self.pages_t.append(torch.zeros(num_blocks, int(m["kv_rank"]), PAGE, dtype=dt, device=dev)
+                                if own and hops.latent_mfma_ok(pages[-1], int(m["kv_rank"]), int(m["rot_dim"]))
+                                else None)
             shift.append(torch.zeros(num_slots, d, dtype=torch.float32, device=dev) if lw.shift is not None else None)
             if lw.type == "mamba2":
                 Hh, P, N, G = (int(m[k]) for k in ("heads", "vdim", "state", "groups"))
@@ -430,14 +452,16 @@ class BuduraxLM:
         H, D, rd, vd, R = (int(mm[k]) for k in ("heads", "dim", "rot_dim", "vdim", "kv_rank"))
         T, dt, dev = h.shape[0], self.dtype, self.device
         qgd = F.linear(h, lw.qgd)  # [q heads (dim | rot) | output gate | latent, shared rotary key]
-        cache = pages[i if lw.kv_from is None else int(lw.kv_from)]
+        src = i if lw.kv_from is None else int(lw.kv_from)
+        cache, cache_t = pages[src], self.pages_t[src]
         q_rot = torch.empty(T, H, rd, dtype=dt, device=dev)
         hops.latent_prep(qgd, H, D, rd, R, lw.dkv_off, lw.dkv_norm, self.cfg.norm_eps, inp.positions, lw.cos_sin,
-                         lw.rot_dims, cache, inp.slot_mapping, q_rot)
+                         lw.rot_dims, cache, inp.slot_mapping, q_rot, cache_t if lw.kv_from is None else None)
         q_u = qgd[:, :H * (D + rd)].view(T, H, D + rd)[:, :, :D].transpose(0, 1)  # [H, T, dim] (strided view)
         q_lat = torch.bmm(q_u, lw.uk_h)                                           # [H, T, R]
         o_lat = torch.empty(H, T, R, dtype=dt, device=dev)
-        hops.latent_attn(q_lat, q_rot, cache, m.block_tables, m.tok_seg, m.seg, inp.positions, lw.scale, o_lat)
+        hops.latent_attn(q_lat, q_rot, cache, m.block_tables, m.tok_seg, m.seg, inp.positions, lw.scale, o_lat,
+                         cache_t, m.tiles.get(hops.tile_tokens(H)))
         a = torch.bmm(o_lat, lw.uv_ht)                                            # [H, T, vdim]
         ao = torch.empty(T, H * vd, dtype=dt, device=dev)
         hops.sigmoid_mul(a, qgd[:, lw.g_off:lw.g_off + H * vd], ao)

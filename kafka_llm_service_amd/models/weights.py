@@ -280,7 +280,9 @@ def build_model(cfg: ModelConfig, device, tp: int = 1, tp_rank: int = 0, seed: i
                              max_positions=max_positions)
         if weights:
             return bx.load_checkpoint(model, weights)
-        return model.load_tensors(bx.random_tensors(cfg, seed))
+        # small models (and every test) draw on the CPU; large ones directly on the device
+        big = cfg.num_params() > 2e8 and torch.device(device).type == "cuda"
+        return model.load_tensors(bx.random_tensors(cfg, seed, device=device if big else "cpu"))
     if dtype not in (None, torch.bfloat16):
         raise ValueError(f"{cfg.arch} models run in bfloat16 only")
     model = TransformerLM(cfg, device, tp=tp, tp_rank=tp_rank, max_positions=max_positions)

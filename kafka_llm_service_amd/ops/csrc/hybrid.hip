@@ -191,7 +191,8 @@ __global__ __launch_bounds__(NT) void latent_prep_kernel(const AT* __restrict__ 
                                                          int R, int dkv_off, const AT* __restrict__ dkv_w, float eps,
                                                          const int64_t* __restrict__ positions,
                                                          const float* __restrict__ cos_sin, int dims,
-                                                         AT* __restrict__ cache, const int64_t* __restrict__ slots,
+                                                         AT* __restrict__ cache, AT* __restrict__ cache_t,
+                                                         int page, const int64_t* __restrict__ slots,
                                                          AT* __restrict__ q_rot) {
   __shared__ float red[NT / 64];
   const int64_t t = blockIdx.x;
@@ -212,7 +213,14 @@ __global__ __launch_bounds__(NT) void latent_prep_kernel(const AT* __restrict__ 
   const float r = inv_sqrt(block_sum<NT>(s, red) / (float)R + eps);
   if (slot < 0) return;
   AT* dst = cache + slot * (R + rd);
-  for (int i = threadIdx.x; i < R; i += NT) stf(dst + i, ldf(lat + i) * r * ldf(dkv_w + i));
+  // the latent part a second time, page-wise transposed [page][dim][token in page]: the MFMA attention kernel reads
+  // its value operand (contraction over keys) from it with 16-byte loads
+  AT* dst_t = cache_t != nullptr ? cache_t + (slot / page) * (int64_t)R * page + (slot % page) : nullptr;
+  for (int i = threadIdx.x; i < R; i += NT) {
+    const float v = ldf(lat + i) * r * ldf(dkv_w + i);
+    stf(dst + i, v);
+    if (dst_t != nullptr) stf(dst_t + (int64_t)i * page, v);
+  }
   for (int j = threadIdx.x; j < rd; j += NT) stf(dst + R + j, rot_elem(lat + R, j, dims, cs));
 }
 
@@ -328,6 +336,147 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(const AT* __restrict__
         const int dim = lane + 64 * c;
         if (dim < R) stf(out + (int64_t)(h0 + r) * o_h + (int64_t)t * o_t + dim, acc[r][c] * inv);
       }
+    }
+  }
+}
+
+
+// ---- latent attention on the matrix cores (bf16) -------------------------------------------------------------------
+// One workgroup (4 waves) per tile of 32 query rows = (token, head) pairs that read the same sequence: all heads of
+// floor(32 / H) consecutive tokens of a segment, or 32 heads of one token. Keys go by in blocks of 128:
+//   scores   wave w takes keys 32 w .. 32 w + 31 of the block: S = Q K^T as Dk / 16 MFMA steps (32x32x16), the Q tile
+//            read from LDS, the key rows straight from the paged cache (lane = key, 16 bytes per step);
+//   softmax  row maxima within the wave by lane exchange and across the four waves through LDS; P = 2^(S - m) goes to
+//            LDS as bf16; the row sums stay per lane and are combined once at the end;
+//   values   wave w owns output columns [32 TW w, 32 TW (w + 1)) of the latent: O += P V with V read from the
+//            page-transposed latent copy (lane = column, 8 consecutive keys = 16 bytes), one page per MFMA step.
+// Scores, maxima, sums and the accumulators are fp32. Needs 16-token pages, kv_rank % 32 == 0, rot_dim % 16 == 0.
+template <int TW>
+__global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
+    const bf16* __restrict__ q_lat, int64_t ql_h, int64_t ql_t, const bf16* __restrict__ q_rot, int64_t qr_t,
+    int64_t qr_h, const bf16* __restrict__ cache, const bf16* __restrict__ cache_t, int R, int rd,
+    const int* __restrict__ bt, int bt_stride, const int* __restrict__ items, const int64_t* __restrict__ positions,
+    float scale_log2e, bf16* __restrict__ out, int64_t o_h, int64_t o_t, int H) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int Dk = R + rd, nks = Dk >> 4, qstride = Dk + 8;
+  bf16* Qs = reinterpret_cast<bf16*>(smem);                 // [32][Dk + 8]
+  bf16* Ps = Qs + 32 * qstride;                             // [32][128 + 8]
+  float* mloc = reinterpret_cast<float*>(Ps + 32 * 136);    // [4][32]
+  int* prow_s = reinterpret_cast<int*>(mloc + 128);         // [32]
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, lr = lane & 31, lh = lane >> 5;
+  const int t0 = items[4 * blockIdx.x], ntok = items[4 * blockIdx.x + 1], sg = items[4 * blockIdx.x + 2];
+  const int h0 = blockIdx.y * 32;
+  const int hpr = min(H - h0, 32);
+  const int nrows = ntok * hpr;
+  // stage Q (zeros for rows beyond the tile) and the rows' positions
+  for (int i = threadIdx.x; i < 32 * (Dk >> 3); i += 256) {
+    const int r = i / (Dk >> 3), d0 = (i - r * (Dk >> 3)) << 3;
+    bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (r < nrows) {
+      const int64_t t = t0 + r / hpr, h = h0 + r % hpr;
+      v = d0 < R ? load_bf16x8(q_lat + h * ql_h + t * ql_t + d0) : load_bf16x8(q_rot + t * qr_t + h * qr_h + (d0 - R));
+    }
+    store_bf16x8(Qs + r * qstride + d0, v);
+  }
+  if (threadIdx.x < 32) prow_s[threadIdx.x] = threadIdx.x < nrows ? (int)positions[t0 + threadIdx.x / hpr] : 0;
+  __syncthreads();
+  const int maxpos = (int)positions[t0 + ntok - 1];
+  int prow[16];
+  float m[16], lsum[16];
+  f32x16 O[TW];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    prow[i] = prow_s[(i & 3) + 8 * (i >> 2) + 4 * lh];
+    m[i] = -INFINITY;
+    lsum[i] = 0.f;
+  }
+#pragma unroll
+  for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) O[tw][i] = 0.f;
+  const int* btr = bt + (int64_t)sg * bt_stride;
+  const int nblocks = (maxpos >> 7) + 1;
+  for (int kb = 0; kb < nblocks; ++kb) {
+    // ---- scores of this wave's 32 keys
+    const int key = kb * 128 + 32 * w + lr;
+    const int kc = min(key, maxpos);  // keys past the tile's last position: a valid row, masked below
+    const bf16* krow = cache + ((int64_t)btr[kc >> 4] * 16 + (kc & 15)) * Dk + 8 * lh;
+    const bf16* qrow = Qs + lr * qstride + 8 * lh;
+    f32x16 S;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) S[i] = 0.f;
+    const bool any = kb * 128 + 32 * w <= maxpos;  // (uniform per wave)
+    if (any) {
+#pragma unroll 4
+      for (int ks = 0; ks < nks; ++ks) S = mfma32(load_bf16x8(qrow + 16 * ks), load_bf16x8(krow + 16 * ks), S);
+    }
+    float s[16], mx[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      s[i] = (any && key <= prow[i]) ? S[i] * scale_log2e : -INFINITY;
+      float v = s[i];
+#pragma unroll
+      for (int o = 16; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+      mx[i] = v;
+    }
+    if (lr == 0) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) mloc[w * 32 + (i & 3) + 8 * (i >> 2) + 4 * lh] = mx[i];
+    }
+    __syncthreads();
+    float corr[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int r = (i & 3) + 8 * (i >> 2) + 4 * lh;
+      const float mn = fmaxf(fmaxf(m[i], fmaxf(mloc[r], mloc[32 + r])), fmaxf(mloc[64 + r], mloc[96 + r]));
+      corr[i] = fast_exp2(m[i] - mn);  // first block: m = -inf, mn finite (key 0 is visible to every row) -> 0
+      const float p = fast_exp2(s[i] - mn);
+      lsum[i] = lsum[i] * corr[i] + p;
+      m[i] = mn;
+      Ps[r * 136 + 32 * w + lr] = (bf16)p;
+    }
+#pragma unroll
+    for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) O[tw][i] *= corr[i];
+    __syncthreads();
+    // ---- values: one page (16 keys) per step
+#pragma unroll 2
+    for (int kk = 0; kk < 8; ++kk) {
+      if ((kb * 8 + kk) * 16 > maxpos) break;  // (uniform) pages past the last position
+      const bf16x8 a = load_bf16x8(Ps + lr * 136 + 16 * kk + 8 * lh);
+      const bf16* vp = cache_t + (int64_t)btr[kb * 8 + kk] * R * 16 + 8 * lh;
+#pragma unroll
+      for (int tw = 0; tw < TW; ++tw) {
+        const int ct = w * TW + tw;
+        if (ct * 32 < R) O[tw] = mfma32(a, load_bf16x8(vp + (int64_t)(ct * 32 + lr) * 16), O[tw]);
+      }
+    }
+    __syncthreads();
+  }
+  // ---- row sums: across the lanes of a half, then across the waves
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    float v = lsum[i];
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    lsum[i] = v;
+  }
+  if (lr == 0) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) mloc[w * 32 + (i & 3) + 8 * (i >> 2) + 4 * lh] = lsum[i];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int r = (i & 3) + 8 * (i >> 2) + 4 * lh;
+    if (r >= nrows) continue;
+    const float inv = 1.0f / (mloc[r] + mloc[32 + r] + mloc[64 + r] + mloc[96 + r]);
+    const int64_t t = t0 + r / hpr, h = h0 + r % hpr;
+#pragma unroll
+    for (int tw = 0; tw < TW; ++tw) {
+      const int ct = w * TW + tw;
+      if (ct * 32 < R) out[h * o_h + t * o_t + ct * 32 + lr] = (bf16)(O[tw][i] * inv);
     }
   }
 }
@@ -554,11 +703,12 @@ hipError_t kafka_hy_side_dwa(int f32, float* x, const void* y, int64_t ys, const
 
 hipError_t kafka_hy_latent_prep(int f32, const void* qgd, int64_t qs, int T, int H, int dim, int rd, int R, int dkv_off,
                                 const void* dkv_w, float eps, const int64_t* positions, const float* cos_sin, int dims,
-                                void* cache, const int64_t* slots, void* q_rot, hipStream_t st) {
+                                void* cache, void* cache_t, int page, const int64_t* slots, void* q_rot,
+                                hipStream_t st) {
   if (T <= 0) return hipSuccess;
   DISPATCH_AT(f32, latent_prep_kernel<AT><<<T, NT, 0, st>>>((const AT*)qgd, qs, H, dim, rd, R, dkv_off,
                                                            (const AT*)dkv_w, eps, positions, cos_sin, dims, (AT*)cache,
-                                                           slots, (AT*)q_rot));
+                                                           (AT*)cache_t, page, slots, (AT*)q_rot));
   return hipGetLastError();
 }
 
@@ -594,6 +744,34 @@ hipError_t kafka_hy_latent_attn(int f32, const void* q_lat, int64_t ql_h, int64_
     else if (Dk <= 640) a(latent_attn_kernel<AT, 10, RPW, 2>);
     else return hipErrorInvalidValue;
   });
+  return hipGetLastError();
+}
+
+// bf16 shapes the matrix-core kernel takes (else the per-wave kernel above runs)
+int kafka_hy_latent_mfma_ok(int page, int R, int rd) {
+  return page == 16 && R % 32 == 0 && rd % 16 == 0 && R >= 32 && R <= 512 && R + rd <= 640;
+}
+
+hipError_t kafka_hy_latent_attn_mfma(const void* q_lat, int64_t ql_h, int64_t ql_t, const void* q_rot, int64_t qr_t,
+                                     int64_t qr_h, const void* cache, const void* cache_t, int R, int rd,
+                                     const int* bt, int bt_stride, const int* items, int n_items,
+                                     const int64_t* positions, float scale, void* out, int64_t o_h, int64_t o_t, int H,
+                                     hipStream_t st) {
+  if (n_items <= 0) return hipSuccess;
+  if (!kafka_hy_latent_mfma_ok(16, R, rd)) return hipErrorInvalidValue;
+  const int Dk = R + rd;
+  const size_t lds = (size_t)32 * (Dk + 8) * 2 + 32 * 136 * 2 + 128 * 4 + 32 * 4;
+  const dim3 grid((unsigned)n_items, (unsigned)((H + 31) / 32));
+  const float sl = scale * 1.4426950408889634f;
+  const int tw = (R / 32 + 3) / 4;
+  auto a = [&](auto k) {
+    k<<<grid, 256, lds, st>>>((const bf16*)q_lat, ql_h, ql_t, (const bf16*)q_rot, qr_t, qr_h, (const bf16*)cache,
+                              (const bf16*)cache_t, R, rd, bt, bt_stride, items, positions, sl, (bf16*)out, o_h, o_t, H);
+  };
+  if (tw == 1) a(latent_attn_mfma_kernel<1>);
+  else if (tw == 2) a(latent_attn_mfma_kernel<2>);
+  else if (tw == 3) a(latent_attn_mfma_kernel<3>);
+  else a(latent_attn_mfma_kernel<4>);
   return hipGetLastError();
 }
 

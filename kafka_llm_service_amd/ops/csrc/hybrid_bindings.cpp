@@ -19,7 +19,14 @@ hipError_t kafka_hy_side_dwa(int f32, float* x, const void* y, int64_t ys, const
                              int layer, const float* dwa, int64_t T, int d, hipStream_t st);
 hipError_t kafka_hy_latent_prep(int f32, const void* qgd, int64_t qs, int T, int H, int dim, int rd, int R, int dkv_off,
                                 const void* dkv_w, float eps, const int64_t* positions, const float* cos_sin, int dims,
-                                void* cache, const int64_t* slots, void* q_rot, hipStream_t st);
+                                void* cache, void* cache_t, int page, const int64_t* slots, void* q_rot,
+                                hipStream_t st);
+int kafka_hy_latent_mfma_ok(int page, int R, int rd);
+hipError_t kafka_hy_latent_attn_mfma(const void* q_lat, int64_t ql_h, int64_t ql_t, const void* q_rot, int64_t qr_t,
+                                     int64_t qr_h, const void* cache, const void* cache_t, int R, int rd,
+                                     const int* bt, int bt_stride, const int* items, int n_items,
+                                     const int64_t* positions, float scale, void* out, int64_t o_h, int64_t o_t, int H,
+                                     hipStream_t st);
 hipError_t kafka_hy_sigmoid_mul(int f32, const void* a, int64_t a_h, int64_t a_t, const void* g, int64_t gs, void* out,
                                 int64_t T, int H, int vd, hipStream_t st);
 int kafka_hy_latent_attn_max_dk();
@@ -183,7 +190,7 @@ void side_dwa(at::Tensor x, OptT y, OptT sw, double eps, OptT stack, int64_t lay
 
 void latent_prep(at::Tensor qgd, int64_t H, int64_t dim, int64_t rd, int64_t R, int64_t dkv_off, OptT dkv_w, double eps,
                  at::Tensor positions, at::Tensor cos_sin, int64_t dims, at::Tensor cache, at::Tensor slots,
-                 at::Tensor q_rot) {
+                 at::Tensor q_rot, OptT cache_t) {
   rows2d(qgd, "qgd");
   const int f32 = act_f32(qgd);
   same_act(f32, {&cache, &q_rot});
@@ -199,6 +206,14 @@ void latent_prep(at::Tensor qgd, int64_t H, int64_t dim, int64_t rd, int64_t R, 
                   q_rot.size(2) == rd, "latent_prep: q_rot [T, H, rot_dim]");
   TORCH_CHECK(cache.is_contiguous() && cache.dim() == 3 && cache.size(2) == R + rd, "latent_prep: cache [pages, page, "
               "kv_rank + rot_dim]");
+  void* ctp = nullptr;
+  if (cache_t.has_value()) {
+    same_act(f32, {&*cache_t});
+    TORCH_CHECK(cache_t->is_contiguous() && cache_t->dim() == 3 && cache_t->size(0) == cache.size(0) &&
+                    cache_t->size(1) == R && cache_t->size(2) == cache.size(1),
+                "latent_prep: transposed latent copy [pages, kv_rank, page]");
+    ctp = cache_t->data_ptr();
+  }
   const void* wp = nullptr;
   if (dkv_off >= 0) {
     TORCH_CHECK(dkv_w.has_value() && dkv_off + R + rd <= qgd.size(1), "latent_prep: latent columns");
@@ -207,7 +222,8 @@ void latent_prep(at::Tensor qgd, int64_t H, int64_t dim, int64_t rd, int64_t R, 
   }
   HY_HIP(kafka_hy_latent_prep(f32, qgd.data_ptr(), qgd.stride(0), (int)T, (int)H, (int)dim, (int)rd, (int)R,
                               (int)dkv_off, wp, (float)eps, positions.data_ptr<int64_t>(), cos_sin.data_ptr<float>(),
-                              (int)dims, cache.data_ptr(), slots.data_ptr<int64_t>(), q_rot.data_ptr(), stream()));
+                              (int)dims, cache.data_ptr(), ctp, (int)cache.size(1), slots.data_ptr<int64_t>(),
+                              q_rot.data_ptr(), stream()));
 }
 
 void sigmoid_mul(at::Tensor a, at::Tensor g, at::Tensor out) {
@@ -243,6 +259,38 @@ void latent_attn(at::Tensor q_lat, at::Tensor q_rot, at::Tensor cache, at::Tenso
                               bt.data_ptr<int>(), (int)bt.stride(0), tok_seg.data_ptr<int>(),
                               positions.data_ptr<int64_t>(), (float)scale, out.data_ptr(), out.stride(0), out.stride(1),
                               (int)T, (int)H, stream()));
+}
+
+// the matrix-core kernel: items int32 [n, 4] = (first row, tokens, segment, 0), each at most 32 (token, head) rows of
+// one segment (or one token, whose heads go 32 at a time over grid.y)
+void latent_attn_mfma(at::Tensor q_lat, at::Tensor q_rot, at::Tensor cache, at::Tensor cache_t, at::Tensor bt,
+                      at::Tensor items, int64_t tile_tokens, at::Tensor positions, double scale, at::Tensor out) {
+  for (const at::Tensor* t : {&q_lat, &q_rot, &cache, &cache_t, &out})
+    TORCH_CHECK(t->is_cuda() && t->scalar_type() == at::kBFloat16, "latent_attn_mfma: bf16 GPU tensors");
+  TORCH_CHECK(q_lat.dim() == 3 && q_lat.stride(2) == 1 && out.dim() == 3 && out.stride(2) == 1 && q_rot.dim() == 3 &&
+                  q_rot.stride(2) == 1, "latent_attn_mfma: q_lat / out [H, T, R], q_rot [T, H, rot_dim]");
+  const int64_t H = q_lat.size(0), T = q_lat.size(1), R = q_lat.size(2), rd = q_rot.size(2);
+  TORCH_CHECK(q_rot.size(0) == T && q_rot.size(1) == H && out.size(0) == H && out.size(1) == T && out.size(2) == R,
+              "latent_attn_mfma: shapes");
+  TORCH_CHECK(cache.is_contiguous() && cache.dim() == 3 && cache.size(2) == R + rd && cache_t.is_contiguous() &&
+                  cache_t.dim() == 3 && cache_t.size(0) == cache.size(0) && cache_t.size(1) == R &&
+                  cache_t.size(2) == cache.size(1), "latent_attn_mfma: cache [pages, 16, R + rd] and [pages, R, 16]");
+  TORCH_CHECK(kafka_hy_latent_mfma_ok((int)cache.size(1), (int)R, (int)rd), "latent_attn_mfma: sizes not supported");
+  // 16-byte loads: every row start must be a multiple of 8 elements
+  TORCH_CHECK(q_lat.stride(0) % 8 == 0 && q_lat.stride(1) % 8 == 0 && q_rot.stride(0) % 8 == 0 &&
+                  q_rot.stride(1) % 8 == 0 && (reinterpret_cast<uintptr_t>(q_lat.data_ptr()) & 15) == 0 &&
+                  (reinterpret_cast<uintptr_t>(q_rot.data_ptr()) & 15) == 0, "latent_attn_mfma: query alignment");
+  TORCH_CHECK(tile_tokens >= 1 && tile_tokens * std::min<int64_t>(H, 32) <= 32 && (H <= 32 || tile_tokens == 1),
+              "latent_attn_mfma: a tile holds at most 32 (token, head) rows");
+  TORCH_CHECK(bt.is_cuda() && bt.scalar_type() == at::kInt && bt.dim() == 2 && bt.stride(1) == 1 && items.is_cuda() &&
+                  items.scalar_type() == at::kInt && items.is_contiguous() && items.dim() == 2 && items.size(1) == 4 &&
+                  positions.is_cuda() && positions.scalar_type() == at::kLong && positions.is_contiguous() &&
+                  positions.numel() == T, "latent_attn_mfma: block tables / items / positions");
+  HY_HIP(kafka_hy_latent_attn_mfma(q_lat.data_ptr(), q_lat.stride(0), q_lat.stride(1), q_rot.data_ptr(),
+                                   q_rot.stride(0), q_rot.stride(1), cache.data_ptr(), cache_t.data_ptr(), (int)R,
+                                   (int)rd, bt.data_ptr<int>(), (int)bt.stride(0), items.data_ptr<int>(),
+                                   (int)items.size(0), positions.data_ptr<int64_t>(), (float)scale, out.data_ptr(),
+                                   out.stride(0), out.stride(1), (int)H, stream()));
 }
 
 void conv_silu(at::Tensor proj, int64_t c0, at::Tensor w, at::Tensor b, at::Tensor tok_seg, at::Tensor seg,
@@ -314,7 +362,11 @@ void kafka_bind_hybrid(pybind11::module_& m) {
   m.def("hy_gelu_mul", &gelu_mul);
   m.def("hy_side_gate", &side_gate);
   m.def("hy_side_dwa", &side_dwa);
-  m.def("hy_latent_prep", &latent_prep);
+  m.def("hy_latent_prep", &latent_prep, py::arg("qgd"), py::arg("H"), py::arg("dim"), py::arg("rd"), py::arg("R"),
+        py::arg("dkv_off"), py::arg("dkv_w"), py::arg("eps"), py::arg("positions"), py::arg("cos_sin"),
+        py::arg("dims"), py::arg("cache"), py::arg("slots"), py::arg("q_rot"), py::arg("cache_t") = py::none());
+  m.def("hy_latent_attn_mfma", &latent_attn_mfma);
+  m.def("hy_latent_mfma_ok", [](int page, int R, int rd) { return kafka_hy_latent_mfma_ok(page, R, rd) != 0; });
   m.def("hy_sigmoid_mul", &sigmoid_mul);
   m.def("hy_latent_attn", &latent_attn);
   m.def("hy_conv_silu", &conv_silu);

@@ -71,19 +71,49 @@ def side_dwa(x, y, side_w, eps, stack, layer: int, dwa) -> None:
 
 
 def latent_prep(qgd, H, dim, rd, R, dkv_off, dkv_w, eps, positions, cos_sin, rot_dims, cache, slot_mapping,
-                q_rot) -> None:
+                q_rot, cache_t=None) -> None:
+    """RMS norm of the latent and rotary on the shared key part of the fused projection row -> the row's cache slot
+    ([latent | rotated key]; with ``cache_t`` [pages, kv_rank, page] also the latent page-wise transposed, the value
+    operand of the matrix-core attention kernel); rotary on every head's query part -> ``q_rot``."""
     if _gpu(qgd):
         ext().hy_latent_prep(qgd, int(H), int(dim), int(rd), int(R), int(dkv_off), dkv_w, float(eps), positions,
-                             cos_sin, int(rot_dims), cache, slot_mapping, q_rot)
+                             cos_sin, int(rot_dims), cache, slot_mapping, q_rot, cache_t)
     else:
         ref.latent_prep(qgd, H, dim, rd, R, dkv_off, dkv_w, eps, positions, cos_sin, rot_dims, cache, slot_mapping,
                         q_rot)
+        if cache_t is not None and dkv_off >= 0:
+            ok = slot_mapping >= 0
+            page = cache.shape[1]
+            sl = slot_mapping[ok].long()
+            cache_t[sl // page, :, sl % page] = cache.view(-1, R + rd)[sl][:, :R]
 
 
-def latent_attn(q_lat, q_rot, cache, block_tables, tok_seg, seg, positions, scale, out) -> None:
-    """Causal softmax attention of every row's heads over its sequence's cached [latent | rotated key] rows."""
+MFMA_ROWS = 32  # (token, head) rows of one tile of the matrix-core attention kernel
+
+
+def latent_mfma_ok(cache: torch.Tensor, R: int, rd: int) -> bool:
+    """bf16 GPU caches of sizes the matrix-core kernel takes (16-token pages, kv_rank % 32 == 0, rot_dim % 16 == 0)."""
+    return cache.is_cuda and cache.dtype == torch.bfloat16 and bool(ext().hy_latent_mfma_ok(cache.shape[1], R, rd))
+
+
+def tile_tokens(heads: int) -> int:
+    """Tokens per attention tile: as many whole tokens (all their heads) as fit 32 rows, at least one."""
+    return max(1, MFMA_ROWS // heads)
+
+
+def latent_attn(q_lat, q_rot, cache, block_tables, tok_seg, seg, positions, scale, out, cache_t=None,
+                tiles=None) -> None:
+    """Causal softmax attention of every row's heads over its sequence's cached [latent | rotated key] rows:
+    out[h, t] = sum_j softmax_j((q_lat[h, t] . c_j + q_rot[t, h] . k_j) scale) c_j over the keys j <= position[t].
+    With the transposed latent copy ``cache_t`` and ``tiles`` (int32 [n, 4] = (first row, tokens, segment, 0), at
+    most ``tile_tokens(H)`` tokens of one segment each) bf16 runs on the matrix cores; else one wave per (row, 4
+    heads) on the vector units (fp32, odd sizes)."""
     if _gpu(q_lat):
-        ext().hy_latent_attn(q_lat, q_rot, cache, block_tables, tok_seg, positions, float(scale), out)
+        if cache_t is not None and tiles is not None and q_lat.dtype == torch.bfloat16:
+            ext().hy_latent_attn_mfma(q_lat, q_rot, cache, cache_t, block_tables, tiles, tile_tokens(q_lat.shape[0]),
+                                      positions, float(scale), out)
+        else:
+            ext().hy_latent_attn(q_lat, q_rot, cache, block_tables, tok_seg, positions, float(scale), out)
     else:
         ref.latent_attn(q_lat, q_rot, cache, block_tables, tok_seg, seg, positions, scale, out)
 

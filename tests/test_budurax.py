@@ -254,6 +254,92 @@ def test_latent_attention_single_keys(device, R, rd, H):
         assert torch.allclose(out[:, i].cpu().double(), want, atol=1e-5), i
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("R,rd,H", [(64, 16, 3), (128, 32, 6), (256, 16, 32), (512, 64, 40), (96, 16, 1), (32, 48, 9)])
+def test_latent_attention_matrix_cores(R, rd, H):
+    """The bf16 matrix-core kernel: a 40-token portion of a 150-token sequence beside another sequence's single
+    token. Every row's query singles out one key - the first keys, both sides of page and 128-key block borders, the
+    row's own position and the one before - and must return that key's latent; then diffuse queries against the plain
+    softmax."""
+    device = "cuda:0"
+    torch.manual_seed(5)
+    nA, nB, page = 150, 37, 16
+    kvA = torch.nn.functional.normalize(torch.randn(nA, R + rd), dim=-1).bfloat16()
+    kvB = torch.nn.functional.normalize(torch.randn(nB, R + rd), dim=-1).bfloat16()
+    cache = torch.zeros(24, page, R + rd, dtype=torch.bfloat16, device=device)
+    orderA, orderB = [7, 2, 9, 4, 0, 11, 20, 13, 5, 16], [3, 21, 8]
+    bt = torch.zeros(2, 16, dtype=torch.int32, device=device)
+    bt[0, :len(orderA)] = torch.tensor(orderA)
+    bt[1, :len(orderB)] = torch.tensor(orderB)
+    flat = cache.view(-1, R + rd)
+    for kv, order in ((kvA, orderA), (kvB, orderB)):
+        for j in range(kv.shape[0]):
+            flat[order[j // page] * page + j % page] = kv[j].to(device)
+    cache_t = cache[:, :, :R].transpose(1, 2).contiguous()
+    posA = list(range(110, 150))
+    pos = posA + [nB - 1]
+    T = len(pos)
+    cands = [0, 1, 15, 16, 17, 31, 32, 111, 112, 127, 128, 129]
+    targets = [[c for c in cands + [p - 1, p] if c <= p][(i * 5) % len([c for c in cands + [p - 1, p] if c <= p])]
+               for i, p in enumerate(posA)] + [nB - 1]
+    kvs = [kvA] * len(posA) + [kvB]
+    tt = hops.tile_tokens(H)
+    tiles = [(a, min(tt, 40 - a), 0, 0) for a in range(0, 40, tt)] + [(40, 1, 1, 0)]
+    tiles = torch.tensor(tiles, dtype=torch.int32, device=device)
+    seg, ts = _seg(device, [(40, 110, 0), (1, nB - 1, 1)])
+    positions = torch.tensor(pos, device=device)
+    q = torch.stack([kvs[i][j].float() for i, j in enumerate(targets)]) * 80.0
+    q_lat = q[:, :R][None].repeat(H, 1, 1).bfloat16().contiguous().to(device)
+    q_rot = q[:, R:][:, None].repeat(1, H, 1).bfloat16().contiguous().to(device)
+    out = torch.empty(H, T, R, dtype=torch.bfloat16, device=device)
+    hops.latent_attn(q_lat, q_rot, cache, bt, ts, seg, positions, 1.0, out, cache_t, tiles)
+    for i, j in enumerate(targets):
+        assert torch.allclose(out[:, i].float().cpu(), kvs[i][j, :R].float().expand(H, R), atol=6e-3), (i, pos[i], j)
+    q_lat = torch.randn(H, T, R).bfloat16()
+    q_rot = torch.randn(T, H, rd).bfloat16()
+    hops.latent_attn(q_lat.to(device), q_rot.to(device), cache, bt, ts, seg, positions, 0.4, out, cache_t, tiles)
+    ref = torch.empty(H, T, R, dtype=torch.bfloat16, device=device)
+    hops.latent_attn(q_lat.to(device), q_rot.to(device), cache, bt, ts, seg, positions, 0.4, ref)  # vector kernel
+    for i, p in enumerate(pos):
+        kv = kvs[i][:p + 1].double()
+        s = (q_lat[:, i].double() @ kv[:, :R].T + q_rot[i].double() @ kv[:, R:].T) * 0.4
+        want = torch.softmax(s, -1) @ kv[:, :R]
+        assert torch.allclose(out[:, i].double().cpu(), want, atol=3e-3), (i, p)
+        assert torch.allclose(ref[:, i].double().cpu(), want, atol=3e-3), (i, p)
+
+
+def cfg_m():
+    """Sizes the matrix-core attention kernel takes (latent 64, rotary part 16), two attention layers sharing a cache."""
+    ff = {"kind": "dense", "ff": 96}
+    return {"architecture": "Budurax", "vocab": 173, "width": 80, "norm": {"eps": 1e-5}, "token_side": {"dim": 4},
+            "layers": [{"type": "latent_attention", "mixer": _attn(5, 16, 16, 16, 24, 64), "mlp": ff},
+                       {"type": "mamba2", "mixer": _mamba(2, 16, 8, 1, 2, 4), "mlp": ff},
+                       {"type": "latent_attention", "mixer": _attn(5, 16, 16, 16, 24, 64, kv_from=0), "mlp": ff}]}
+
+
+@pytest.mark.gpu
+def test_matrix_core_attention_in_the_engine():
+    """bf16 on the GPU with an eligible latent size: whole prompt, portions, single tokens and a mixed batch through
+    the matrix-core kernel against the plain model, and against the same engine in fp32 (vector kernel)."""
+    b = Bench(cfg_m(), seed=11, sharpen=2.0)
+    t, u = toks(300, 173, 1), toks(41, 173, 2)
+    eng = b.engine("cuda:0", "bfloat16", blocks=40)
+    assert any(p is not None for p in eng.model.pages_t)
+    assert rel_err(feed_all(eng, "w", t, [300]), b.oracle(t)) < TOL["bfloat16"]
+    assert rel_err(feed_all(eng, "c", t, [130, 2, 61, 1, 1, 1, 40, 1]), b.oracle(t)) < TOL["bfloat16"]
+    got_t, got_u = [], []
+    got_t.append(eng.feed([("t", t[:200], list(range(200)))]))
+    out = eng.feed([("u", u[:40], list(range(40))), ("t", t[200:201], [0])])
+    got_u.append(out[:40])
+    got_t.append(out[40:])
+    out = eng.feed([("t", t[201:], list(range(99))), ("u", u[40:], [0])], ["t", "u"])
+    got_t.append(out[:99])
+    got_u.append(out[99:])
+    assert rel_err(torch.cat(got_t), b.oracle(t)) < TOL["bfloat16"]
+    assert rel_err(torch.cat(got_u), b.oracle(u)) < TOL["bfloat16"]
+    assert eng.kvm.num_free() == 40
+
+
 @pytest.mark.parametrize("device", DEVICES)
 def test_conv_and_scan_portions(device):
     """Convolution tail and state-space state carried over portions of 1, 2, 3 and 7 rows, with another sequence's run
