@@ -20,8 +20,8 @@
 //                   heads), the 64 lanes across the row's dimensions, online softmax, the value pass reusing the key
 //                   registers (the values ARE the latent part of the key row)
 //   conv_silu       causal short convolution + silu with a per-slot tail of raw inputs
-//   ssm_scan        the state-space recurrence, one workgroup per (segment, head), state in registers, B / C / x / dt
-//                   of 8 tokens staged through LDS
+//   ssm_scan        the state-space recurrence, one workgroup per (segment, head, column slice), an 8 x 4 state block
+//                   per thread in registers, B / C / x / dt of the next tokens staged through LDS, double buffered
 //   gated_norm      y * silu(z), RMS norm in groups, weight
 #include "common.h"
 
@@ -40,6 +40,11 @@ __device__ __forceinline__ float sigmoidf(float z) { return 1.0f / (1.0f + expf(
 __device__ __forceinline__ float inv_sqrt(float v) { return 1.0f / sqrtf(v); }
 
 constexpr int NT = 256;
+
+// Workgroup barrier for LDS hand-overs that leaves global loads in flight: __syncthreads() drains vmcnt as well,
+// which would stall on every prefetch issued before it. This wave's LDS reads and writes are complete (lgkmcnt 0)
+// before it arrives.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // mean and 1 / sqrt(var + eps) of an fp32 or AT row
 template <typename XT>
@@ -351,8 +356,10 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(const AT* __restrict__
 //   values   wave w owns output columns [32 TW w, 32 TW (w + 1)) of the latent: O += P V with V read from the
 //            page-transposed latent copy (lane = column, 8 consecutive keys = 16 bytes), one page per MFMA step.
 // Scores, maxima, sums and the accumulators are fp32. Needs 16-token pages, kv_rank % 32 == 0, rot_dim % 16 == 0.
-template <int TW>
-__global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
+constexpr int MFMA_PG = 2048;  // pages of a tile's sequence staged in LDS (32k tokens; later pages read the table)
+
+template <int TW, int NKSC>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void latent_attn_mfma_kernel(
     const bf16* __restrict__ q_lat, int64_t ql_h, int64_t ql_t, const bf16* __restrict__ q_rot, int64_t qr_t,
     int64_t qr_h, const bf16* __restrict__ cache, const bf16* __restrict__ cache_t, int R, int rd,
     const int* __restrict__ bt, int bt_stride, const int* __restrict__ items, const int64_t* __restrict__ positions,
@@ -363,6 +370,8 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
   bf16* Ps = Qs + 32 * qstride;                             // [32][128 + 8]
   float* mloc = reinterpret_cast<float*>(Ps + 32 * 136);    // [4][32]
   int* prow_s = reinterpret_cast<int*>(mloc + 128);         // [32]
+  int* pg_s = prow_s + 32;                                  // [MFMA_PG]: the tile's first pages (no dependent
+                                                            // global load of the block table in front of a key load)
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, lr = lane & 31, lh = lane >> 5;
   const int t0 = items[4 * blockIdx.x], ntok = items[4 * blockIdx.x + 1], sg = items[4 * blockIdx.x + 2];
   const int h0 = blockIdx.y * 32;
@@ -379,8 +388,13 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
     store_bf16x8(Qs + r * qstride + d0, v);
   }
   if (threadIdx.x < 32) prow_s[threadIdx.x] = threadIdx.x < nrows ? (int)positions[t0 + threadIdx.x / hpr] : 0;
-  __syncthreads();
   const int maxpos = (int)positions[t0 + ntok - 1];
+  {
+    const int* btg = bt + (int64_t)sg * bt_stride;
+    const int np = min((maxpos >> 4) + 1, MFMA_PG);
+    for (int i = threadIdx.x; i < np; i += 256) pg_s[i] = btg[i];
+  }
+  lds_barrier();
   int prow[16];
   float m[16], lsum[16];
   f32x16 O[TW];
@@ -396,20 +410,33 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
     for (int i = 0; i < 16; ++i) O[tw][i] = 0.f;
   const int* btr = bt + (int64_t)sg * bt_stride;
   const int nblocks = (maxpos >> 7) + 1;
+  const bf16* qrow = Qs + lr * qstride + 8 * lh;
+  // this wave's key row of a block, all its 16-dim steps in flight at once (one memory round trip per block); the
+  // next block's row is requested right after this block's score MFMAs, so it arrives under the softmax and the
+  // value pass
+  bf16x8 kf[NKSC];
+  auto fetch_keys = [&](int kb) {
+    const int kc = min(kb * 128 + 32 * w + lr, maxpos);  // past the tile's last position: a valid row, masked below
+    const int pi = kc >> 4;
+    const bf16* krow = cache + ((int64_t)(pi < MFMA_PG ? pg_s[pi] : btr[pi]) * 16 + (kc & 15)) * Dk + 8 * lh;
+#pragma unroll
+    for (int ks = 0; ks < NKSC; ++ks)
+      if (ks < nks) kf[ks] = load_bf16x8(krow + 16 * ks);
+  };
+  if (32 * w <= maxpos) fetch_keys(0);
   for (int kb = 0; kb < nblocks; ++kb) {
     // ---- scores of this wave's 32 keys
     const int key = kb * 128 + 32 * w + lr;
-    const int kc = min(key, maxpos);  // keys past the tile's last position: a valid row, masked below
-    const bf16* krow = cache + ((int64_t)btr[kc >> 4] * 16 + (kc & 15)) * Dk + 8 * lh;
-    const bf16* qrow = Qs + lr * qstride + 8 * lh;
     f32x16 S;
 #pragma unroll
     for (int i = 0; i < 16; ++i) S[i] = 0.f;
     const bool any = kb * 128 + 32 * w <= maxpos;  // (uniform per wave)
     if (any) {
-#pragma unroll 4
-      for (int ks = 0; ks < nks; ++ks) S = mfma32(load_bf16x8(qrow + 16 * ks), load_bf16x8(krow + 16 * ks), S);
+#pragma unroll
+      for (int ks = 0; ks < NKSC; ++ks)
+        if (ks < nks) S = mfma32(load_bf16x8(qrow + 16 * ks), kf[ks], S);
     }
+    if (kb + 1 < nblocks && (kb + 1) * 128 + 32 * w <= maxpos) fetch_keys(kb + 1);
     float s[16], mx[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
@@ -423,7 +450,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
 #pragma unroll
       for (int i = 0; i < 16; ++i) mloc[w * 32 + (i & 3) + 8 * (i >> 2) + 4 * lh] = mx[i];
     }
-    __syncthreads();
+    lds_barrier();
     float corr[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
@@ -439,20 +466,32 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
     for (int tw = 0; tw < TW; ++tw)
 #pragma unroll
       for (int i = 0; i < 16; ++i) O[tw][i] *= corr[i];
-    __syncthreads();
+    lds_barrier();
     // ---- values: one page (16 keys) per step
-#pragma unroll 2
-    for (int kk = 0; kk < 8; ++kk) {
-      if ((kb * 8 + kk) * 16 > maxpos) break;  // (uniform) pages past the last position
-      const bf16x8 a = load_bf16x8(Ps + lr * 136 + 16 * kk + 8 * lh);
-      const bf16* vp = cache_t + (int64_t)btr[kb * 8 + kk] * R * 16 + 8 * lh;
 #pragma unroll
-      for (int tw = 0; tw < TW; ++tw) {
-        const int ct = w * TW + tw;
-        if (ct * 32 < R) O[tw] = mfma32(a, load_bf16x8(vp + (int64_t)(ct * 32 + lr) * 16), O[tw]);
+    for (int k0 = 0; k0 < 8; k0 += 4) {
+      bf16x8 vf[4][TW];  // four pages' value operands in flight together
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        if ((kb * 8 + k0 + kk) * 16 > maxpos) break;  // (uniform) pages past the last position
+        const int pi = kb * 8 + k0 + kk;
+        const bf16* vp = cache_t + (int64_t)(pi < MFMA_PG ? pg_s[pi] : btr[pi]) * R * 16 + 8 * lh;
+#pragma unroll
+        for (int tw = 0; tw < TW; ++tw) {
+          const int ct = w * TW + tw;
+          if (ct * 32 < R) vf[kk][tw] = load_bf16x8(vp + (int64_t)(ct * 32 + lr) * 16);
+        }
+      }
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        if ((kb * 8 + k0 + kk) * 16 > maxpos) break;
+        const bf16x8 a = load_bf16x8(Ps + lr * 136 + 16 * (k0 + kk) + 8 * lh);
+#pragma unroll
+        for (int tw = 0; tw < TW; ++tw)
+          if ((w * TW + tw) * 32 < R) O[tw] = mfma32(a, vf[kk][tw], O[tw]);
       }
     }
-    __syncthreads();
+    lds_barrier();
   }
   // ---- row sums: across the lanes of a half, then across the waves
 #pragma unroll
@@ -466,7 +505,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
 #pragma unroll
     for (int i = 0; i < 16; ++i) mloc[w * 32 + (i & 3) + 8 * (i >> 2) + 4 * lh] = lsum[i];
   }
-  __syncthreads();
+  lds_barrier();
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
     const int r = (i & 3) + 8 * (i >> 2) + 4 * lh;
@@ -530,81 +569,154 @@ __global__ void conv_state_kernel(const AT* __restrict__ proj, int64_t ps, int c
   for (int k = 0; k < taps - 1; ++k) st[(int64_t)k * C] = v[k];
 }
 
-constexpr int SCAN_TB = 8;
+// The recurrence S_t = dA_t S_{t-1} + B_t (dt_t x_t)^T, y_t = S_t^T C_t + D x_t of one (segment, head, slice of the
+// head's columns). Thread (tn, tp) keeps an RN x RP block of the state in registers (rows n = tn RN + i, columns
+// p = tp RP + j), so a token costs RN + RN + RP LDS reads for 2 RN RP multiply-adds. The inputs of TB tokens (B, C, x,
+// dt, dA = exp(-exp(A_log) dt)) are staged in LDS, double buffered: the next block's global loads are in flight while
+// this block's tokens are scanned. Each thread's partial y (over its RN rows) goes to LDS and is summed over the TN
+// row groups once per block. A head's columns are independent of each other, so a head may be cut into slices that
+// run as separate workgroups (more workgroups when a step has few sequences).
+constexpr int SCAN_MAXL = 24;  // staged elements a thread fetches per block, at most
 
-template <typename AT, int EPT>
-__global__ void ssm_scan_kernel(const AT* __restrict__ xbc, int64_t xs, const AT* __restrict__ proj, int64_t ps,
+template <typename AT, int RN, int RP>
+__global__ __launch_bounds__(256) void ssm_scan_kernel(const AT* __restrict__ xbc, int64_t xs, const AT* __restrict__ proj, int64_t ps,
                                 int dt_off, const float* __restrict__ dt_bias, const float* __restrict__ A_log,
-                                const float* __restrict__ Dp, int heads, int P, int N, int G, int NG,
-                                const int* __restrict__ seg, float* __restrict__ state, float* __restrict__ y,
-                                int64_t ys) {
+                                const float* __restrict__ Dp, int heads, int P, int N, int G, int TN, int TP, int NPS,
+                                int TB, const int* __restrict__ seg, float* __restrict__ state,
+                                float* __restrict__ y, int64_t ys) {
   extern __shared__ float sm[];
-  const int sgi = blockIdx.x / heads, h = blockIdx.x - sgi * heads;
-  const int q0 = seg[4 * sgi], n = seg[4 * sgi + 1], p0 = seg[4 * sgi + 2], slot = seg[4 * sgi + 3];
-  const int tid = threadIdx.x, nthr = blockDim.x;
-  const int p = tid % P, g = tid / P;
-  const int grp = h / (heads / G);
-  const int inner = heads * P;
-  float S[EPT];
+  const int nthr = blockDim.x, tid = threadIdx.x;
+  const int W = TP * RP;
+  int b = blockIdx.x;
+  const int psl = b % NPS;
+  b /= NPS;
+  const int h = b % heads, sgi = b / heads;
+  const int q0 = seg[4 * sgi], n = seg[4 * sgi + 1], p0s = seg[4 * sgi + 2], slot = seg[4 * sgi + 3];
+  const int tp = tid % TP, tn = tid / TP;
+  const bool active = tn < TN;
+  const int pbase = psl * W, pw = min(W, P - pbase);
+  const int grp = h / (heads / G), inner = heads * P;
+  float S[RN][RP];
   float* st = state + ((int64_t)slot * heads + h) * N * P;
 #pragma unroll
-  for (int k = 0; k < EPT; ++k) {
-    const int nn = g + k * NG;
-    S[k] = (p0 > 0 && nn < N) ? st[(int64_t)nn * P + p] : 0.f;
-  }
-  const float A = -expf(A_log[h]), bias = dt_bias[h], Dh = Dp[h];
-  float* Bs = sm;                    // [TB][N]  (dt * B)
-  float* Cs = Bs + SCAN_TB * N;      // [TB][N]
-  float* xv = Cs + SCAN_TB * N;      // [TB][P]
-  float* dts = xv + SCAN_TB * P;     // [TB]
-  float* dAs = dts + SCAN_TB;        // [TB]
-  float* yp = dAs + SCAN_TB;         // [TB][NG][P]
-  for (int t0 = 0; t0 < n; t0 += SCAN_TB) {
-    const int nt = min(SCAN_TB, n - t0);
-    if (tid < nt) {
-      const float raw = ldf(proj + (int64_t)(q0 + t0 + tid) * ps + dt_off + h) + bias;
-      const float dt = raw > 20.f ? raw : log1pf(expf(raw));  // softplus
-      dts[tid] = dt;
-      dAs[tid] = expf(A * dt);
-    }
-    __syncthreads();
-    for (int i = tid; i < nt * N; i += nthr) {
-      const int tt = i / N, nn = i - tt * N;
-      const AT* row = xbc + (int64_t)(q0 + t0 + tt) * xs + inner + grp * N + nn;
-      Bs[i] = dts[tt] * ldf(row);
-      Cs[i] = ldf(row + (int64_t)G * N);
-    }
-    for (int i = tid; i < nt * P; i += nthr) {
-      const int tt = i / P, pp = i - tt * P;
-      xv[i] = ldf(xbc + (int64_t)(q0 + t0 + tt) * xs + h * P + pp);
-    }
-    __syncthreads();
-    for (int tt = 0; tt < nt; ++tt) {
-      const float dA = dAs[tt], xp = xv[tt * P + p];
-      float a = 0.f;
+  for (int i = 0; i < RN; ++i)
 #pragma unroll
-      for (int k = 0; k < EPT; ++k) {
-        const int nn = g + k * NG;
-        if (nn < N) {
-          S[k] = dA * S[k] + Bs[tt * N + nn] * xp;
-          a += S[k] * Cs[tt * N + nn];
+    for (int j = 0; j < RP; ++j) {
+      const int nn = tn * RN + i, pp = tp * RP + j;
+      S[i][j] = (active && p0s > 0 && nn < N && pp < pw) ? st[(int64_t)nn * P + pbase + pp] : 0.f;
+    }
+  const float A = -expf(A_log[h]), bias = dt_bias[h], Dh = Dp[h];
+  const int NP = TN * RN;               // state rows padded to whole thread blocks: the pad's B and C stay zero in LDS,
+                                        // so the token loop has no bounds tests
+  const int stride = 2 * NP + W + 2;    // per token: B[NP] | C[NP] | x[W] | dt | dA
+  const int per_tok = 2 * N + W + 1;    // fetched per token (dA is derived)
+  const int bufsz = TB * stride;        // two staging buffers at sm[0], sm[bufsz] (plain offsets into the LDS array:
+                                        // a pointer array would decay to generic pointers and flat loads)
+  const int ypo = 2 * bufsz;            // yp [TB][TN][W] at sm[ypo]
+  if (NP != N)
+    for (int i = tid; i < 2 * TB * stride; i += nthr) sm[i] = 0.f;
+  // what this thread fetches of every block: (token in block, element) per slot, fixed for the whole scan
+  int ftok[SCAN_MAXL], fidx[SCAN_MAXL];
+#pragma unroll
+  for (int l = 0; l < SCAN_MAXL; ++l) {
+    const int e = tid + l * nthr;
+    ftok[l] = e / per_tok;
+    fidx[l] = e - ftok[l] * per_tok;
+    if (ftok[l] >= TB) ftok[l] = 1 << 20;  // never fetched
+  }
+  float pre[SCAN_MAXL];
+  auto fetch = [&](int t0) {
+    const int nt = min(TB, n - t0);
+#pragma unroll
+    for (int l = 0; l < SCAN_MAXL; ++l) {
+      if (ftok[l] < nt) {
+        const int idx = fidx[l];
+        const int64_t row = q0 + t0 + ftok[l];
+        // one straight-line load per element (the address is selected, not the load)
+        const AT* xr = xbc + row * xs;
+        const AT* src = idx < N ? xr + inner + grp * N + idx
+                        : idx < 2 * N ? xr + inner + (G + grp) * N + (idx - N)
+                        : idx < 2 * N + W ? xr + h * P + pbase + min(idx - 2 * N, pw - 1)
+                                          : proj + row * ps + dt_off + h;
+        float v = ldf(src);
+        if (idx >= 2 * N && idx < 2 * N + W && idx - 2 * N >= pw) v = 0.f;
+        pre[l] = v;
+      }
+    }
+  };
+  auto stash = [&](int dsto, int t0) {
+    const int nt = min(TB, n - t0);
+#pragma unroll
+    for (int l = 0; l < SCAN_MAXL; ++l) {
+      if (ftok[l] < nt) {
+        const int idx = fidx[l];
+        const int d = dsto + ftok[l] * stride;
+        if (idx == per_tok - 1) {
+          const float raw = pre[l] + bias;
+          const float dt = raw > 20.f ? raw : log1pf(expf(raw));  // softplus
+          sm[d + 2 * NP + W] = dt;
+          sm[d + 2 * NP + W + 1] = expf(A * dt);
+        } else {
+          sm[d + (idx < N ? idx : idx < 2 * N ? NP + (idx - N) : 2 * NP + (idx - 2 * N))] = pre[l];
         }
       }
-      yp[(tt * NG + g) * P + p] = a;
     }
-    __syncthreads();
-    for (int i = tid; i < nt * P; i += nthr) {
-      const int tt = i / P, pp = i - tt * P;
-      float s = 0.f;
-      for (int gg = 0; gg < NG; ++gg) s += yp[(tt * NG + gg) * P + pp];
-      y[(int64_t)(q0 + t0 + tt) * ys + h * P + pp] = s + Dh * xv[i];
-    }
-    __syncthreads();
-  }
+  };
+  lds_barrier();  // (the zero fill)
+  fetch(0);
+  stash(0, 0);
+  lds_barrier();
+  int it = 0;
+  for (int t0 = 0; t0 < n; t0 += TB, ++it) {
+    const int cur = (it & 1) * bufsz;
+    const int nt = min(TB, n - t0);
+    const bool more = t0 + TB < n;
+    if (more) fetch(t0 + TB);  // in flight during the scan below
+    if (active) {
+      for (int tt = 0; tt < nt; ++tt) {
+        const float* r = sm + cur + tt * stride;
+        const float dt = r[2 * NP + W], dA = r[2 * NP + W + 1];
+        float dx[RP], acc[RP], Bv[RN], Cv[RN];
 #pragma unroll
-  for (int k = 0; k < EPT; ++k) {
-    const int nn = g + k * NG;
-    if (nn < N) st[(int64_t)nn * P + p] = S[k];
+        for (int j = 0; j < RP; ++j) {
+          dx[j] = dt * r[2 * NP + tp * RP + j];
+          acc[j] = 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < RN; ++i) {
+          Bv[i] = r[tn * RN + i];
+          Cv[i] = r[NP + tn * RN + i];
+        }
+#pragma unroll
+        for (int i = 0; i < RN; ++i)
+#pragma unroll
+          for (int j = 0; j < RP; ++j) {
+            S[i][j] = dA * S[i][j] + Bv[i] * dx[j];
+            acc[j] += S[i][j] * Cv[i];
+          }
+#pragma unroll
+        for (int j = 0; j < RP; ++j) sm[ypo + (tt * TN + tn) * W + tp * RP + j] = acc[j];
+      }
+    }
+    lds_barrier();
+    for (int e = tid; e < nt * pw; e += nthr) {
+      const int tt = e / pw, pp = e - tt * pw;
+      float s = 0.f;
+#pragma unroll 8
+      for (int g = 0; g < TN; ++g) s += sm[ypo + (tt * TN + g) * W + pp];
+      y[(int64_t)(q0 + t0 + tt) * ys + h * P + pbase + pp] = s + Dh * sm[cur + tt * stride + 2 * NP + pp];
+    }
+    if (more) stash(bufsz - cur, t0 + TB);
+    lds_barrier();
+  }
+  if (active) {
+#pragma unroll
+    for (int i = 0; i < RN; ++i)
+#pragma unroll
+      for (int j = 0; j < RP; ++j) {
+        const int nn = tn * RN + i, pp = tp * RP + j;
+        if (nn < N && pp < pw) st[(int64_t)nn * P + pbase + pp] = S[i][j];
+      }
   }
 }
 
@@ -760,7 +872,7 @@ hipError_t kafka_hy_latent_attn_mfma(const void* q_lat, int64_t ql_h, int64_t ql
   if (n_items <= 0) return hipSuccess;
   if (!kafka_hy_latent_mfma_ok(16, R, rd)) return hipErrorInvalidValue;
   const int Dk = R + rd;
-  const size_t lds = (size_t)32 * (Dk + 8) * 2 + 32 * 136 * 2 + 128 * 4 + 32 * 4;
+  const size_t lds = (size_t)32 * (Dk + 8) * 2 + 32 * 136 * 2 + 128 * 4 + 32 * 4 + MFMA_PG * 4;
   const dim3 grid((unsigned)n_items, (unsigned)((H + 31) / 32));
   const float sl = scale * 1.4426950408889634f;
   const int tw = (R / 32 + 3) / 4;
@@ -768,10 +880,14 @@ hipError_t kafka_hy_latent_attn_mfma(const void* q_lat, int64_t ql_h, int64_t ql
     k<<<grid, 256, lds, st>>>((const bf16*)q_lat, ql_h, ql_t, (const bf16*)q_rot, qr_t, qr_h, (const bf16*)cache,
                               (const bf16*)cache_t, R, rd, bt, bt_stride, items, positions, sl, (bf16*)out, o_h, o_t, H);
   };
-  if (tw == 1) a(latent_attn_mfma_kernel<1>);
-  else if (tw == 2) a(latent_attn_mfma_kernel<2>);
-  else if (tw == 3) a(latent_attn_mfma_kernel<3>);
-  else a(latent_attn_mfma_kernel<4>);
+  const int nks = Dk / 16;
+  if (tw == 1 && nks <= 12) a(latent_attn_mfma_kernel<1, 12>);
+  else if (tw == 1) a(latent_attn_mfma_kernel<1, 40>);
+  else if (tw == 2 && nks <= 24) a(latent_attn_mfma_kernel<2, 24>);
+  else if (tw == 2) a(latent_attn_mfma_kernel<2, 40>);
+  else if (tw == 3) a(latent_attn_mfma_kernel<3, 40>);
+  else if (nks <= 36) a(latent_attn_mfma_kernel<4, 36>);
+  else a(latent_attn_mfma_kernel<4, 40>);
   return hipGetLastError();
 }
 
@@ -789,32 +905,45 @@ hipError_t kafka_hy_conv_silu(int f32, const void* proj, int64_t ps, int c0, con
   return hipGetLastError();
 }
 
-// threads per workgroup = P * NG; 0 when the state does not fit the kernel's register budget
+// launch shape of the scan for a head of N x P state and `work` = segments x heads workgroups before slicing:
+// returns 0 when no shape fits
+struct ScanPlan { int TN, TP, NPS, TB, threads; size_t lds; };
+static int scan_plan(int P, int N, int64_t work, ScanPlan* sp) {
+  constexpr int RN = 8, RP = 4;
+  if (P < 1 || N < 1 || N > 4096 || P > 4096) return 0;
+  const int TN = (N + RN - 1) / RN;
+  if (TN > 256) return 0;
+  int TP = std::max(1, std::min((P + RP - 1) / RP, std::max(1, 256 / TN)));
+  auto slices = [&](int tp) { return (P + tp * RP - 1) / (tp * RP); };
+  while (TP >= 8 && work * slices(TP) < 256) TP /= 2;  // few sequences: narrower slices, more workgroups
+  const int NPS = slices(TP), W = TP * RP;
+  const int threads = std::max(64, (TN * TP + 63) / 64 * 64);
+  if (threads > 256) return 0;
+  for (int TB = 8; TB >= 1; TB /= 2) {
+    const size_t lds = sizeof(float) * ((size_t)2 * TB * (2 * TN * RN + W + 2) + (size_t)TB * TN * W);
+    const int lpt = (TB * (2 * N + W + 1) + threads - 1) / threads;
+    if (lds <= 60 * 1024 && lpt <= 24) {
+      *sp = {TN, TP, NPS, TB, threads, lds};
+      return 1;
+    }
+  }
+  return 0;
+}
+
 int kafka_hy_scan_groups(int P, int N) {
-  if (P < 1 || P > 1024 || N < 1) return 0;
-  int ng = std::max(1, 256 / P);
-  if ((N + ng - 1) / ng > 32) ng = (N + 31) / 32;
-  return P * ng <= 1024 ? ng : 0;
+  ScanPlan sp;
+  return scan_plan(P, N, 1 << 20, &sp) ? sp.threads : 0;
 }
 
 hipError_t kafka_hy_ssm_scan(int f32, const void* xbc, int64_t xs, const void* proj, int64_t ps, int dt_off,
                              const float* dt_bias, const float* A_log, const float* Dp, int heads, int P, int N, int G,
                              const int* seg, int R, float* state, float* y, int64_t ys, hipStream_t st) {
   if (R <= 0) return hipSuccess;
-  const int NG = kafka_hy_scan_groups(P, N);
-  if (NG == 0) return hipErrorInvalidValue;
-  const int ept = (N + NG - 1) / NG;
-  const size_t lds = sizeof(float) * (size_t)(2 * SCAN_TB * N + SCAN_TB * P + 2 * SCAN_TB + SCAN_TB * NG * P);
-  if (lds > 64 * 1024) return hipErrorInvalidValue;
-  DISPATCH_AT(f32, {
-    auto a = [&](auto k) {
-      k<<<R * heads, P * NG, lds, st>>>((const AT*)xbc, xs, (const AT*)proj, ps, dt_off, dt_bias, A_log, Dp, heads, P,
-                                        N, G, NG, seg, state, y, ys);
-    };
-    if (ept <= 8) a(ssm_scan_kernel<AT, 8>);
-    else if (ept <= 16) a(ssm_scan_kernel<AT, 16>);
-    else a(ssm_scan_kernel<AT, 32>);
-  });
+  ScanPlan sp;
+  if (!scan_plan(P, N, (int64_t)R * heads, &sp)) return hipErrorInvalidValue;
+  DISPATCH_AT(f32, ssm_scan_kernel<AT, 8, 4><<<R * heads * sp.NPS, sp.threads, sp.lds, st>>>(
+                       (const AT*)xbc, xs, (const AT*)proj, ps, dt_off, dt_bias, A_log, Dp, heads, P, N, G, sp.TN,
+                       sp.TP, sp.NPS, sp.TB, seg, state, y, ys));
   return hipGetLastError();
 }
 
