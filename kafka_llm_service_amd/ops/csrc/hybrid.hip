@@ -578,11 +578,11 @@ __global__ void conv_state_kernel(const AT* __restrict__ proj, int64_t ps, int c
 // run as separate workgroups (more workgroups when a step has few sequences).
 constexpr int SCAN_MAXL = 24;  // staged elements a thread fetches per block, at most
 
-template <typename AT, int RN, int RP>
+template <typename AT, int RN, int RP, int TB>
 __global__ __launch_bounds__(256) void ssm_scan_kernel(const AT* __restrict__ xbc, int64_t xs, const AT* __restrict__ proj, int64_t ps,
                                 int dt_off, const float* __restrict__ dt_bias, const float* __restrict__ A_log,
                                 const float* __restrict__ Dp, int heads, int P, int N, int G, int TN, int TP, int NPS,
-                                int TB, const int* __restrict__ seg, float* __restrict__ state,
+                                const int* __restrict__ seg, float* __restrict__ state,
                                 float* __restrict__ y, int64_t ys) {
   extern __shared__ float sm[];
   const int nthr = blockDim.x, tid = threadIdx.x;
@@ -673,30 +673,41 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(const AT* __restrict__ xb
     const bool more = t0 + TB < n;
     if (more) fetch(t0 + TB);  // in flight during the scan below
     if (active) {
-      for (int tt = 0; tt < nt; ++tt) {
-        const float* r = sm + cur + tt * stride;
-        const float dt = r[2 * NP + W], dA = r[2 * NP + W + 1];
-        float dx[RP], acc[RP], Bv[RN], Cv[RN];
+      // the block's tokens fully unrolled, the partial outputs kept in registers until the end: no LDS store
+      // sits between the tokens' LDS reads, so the reads of later tokens are issued under the arithmetic of earlier
+      // ones (one wave per SIMD has nothing else to hide LDS latency with)
+      float accs[TB][RP];
 #pragma unroll
-        for (int j = 0; j < RP; ++j) {
-          dx[j] = dt * r[2 * NP + tp * RP + j];
-          acc[j] = 0.f;
-        }
-#pragma unroll
-        for (int i = 0; i < RN; ++i) {
-          Bv[i] = r[tn * RN + i];
-          Cv[i] = r[NP + tn * RN + i];
-        }
-#pragma unroll
-        for (int i = 0; i < RN; ++i)
+      for (int tt = 0; tt < TB; ++tt) {
+        if (tt < nt) {
+          const float* r = sm + cur + tt * stride;
+          const float dt = r[2 * NP + W], dA = r[2 * NP + W + 1];
+          float dx[RP], Bv[RN], Cv[RN];
 #pragma unroll
           for (int j = 0; j < RP; ++j) {
-            S[i][j] = dA * S[i][j] + Bv[i] * dx[j];
-            acc[j] += S[i][j] * Cv[i];
+            dx[j] = dt * r[2 * NP + tp * RP + j];
+            accs[tt][j] = 0.f;
           }
 #pragma unroll
-        for (int j = 0; j < RP; ++j) sm[ypo + (tt * TN + tn) * W + tp * RP + j] = acc[j];
+          for (int i = 0; i < RN; ++i) {
+            Bv[i] = r[tn * RN + i];
+            Cv[i] = r[NP + tn * RN + i];
+          }
+#pragma unroll
+          for (int i = 0; i < RN; ++i)
+#pragma unroll
+            for (int j = 0; j < RP; ++j) {
+              S[i][j] = dA * S[i][j] + Bv[i] * dx[j];
+              accs[tt][j] += S[i][j] * Cv[i];
+            }
+        }
       }
+#pragma unroll
+      for (int tt = 0; tt < TB; ++tt)
+        if (tt < nt) {
+#pragma unroll
+          for (int j = 0; j < RP; ++j) sm[ypo + (tt * TN + tn) * W + tp * RP + j] = accs[tt][j];
+        }
     }
     lds_barrier();
     for (int e = tid; e < nt * pw; e += nthr) {
@@ -717,6 +728,57 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(const AT* __restrict__ xb
         const int nn = tn * RN + i, pp = tp * RP + j;
         if (nn < N && pp < pw) st[(int64_t)nn * P + pbase + pp] = S[i][j];
       }
+  }
+}
+
+// The recurrence for a step of single tokens (every segment one row: a decode step): one workgroup per (segment,
+// head) streams the head's state through once - thread (g, p) owns column p and the rows n = g, g + NG, ... (the
+// state's rows are read and written as consecutive columns: coalesced) - and the NG partial outputs per column are
+// summed through LDS. No staging, no token loop: the state traffic is the whole cost.
+template <typename AT>
+__global__ __launch_bounds__(256) void ssm_step_kernel(const AT* __restrict__ xbc, int64_t xs,
+                                                       const AT* __restrict__ proj, int64_t ps, int dt_off,
+                                                       const float* __restrict__ dt_bias,
+                                                       const float* __restrict__ A_log, const float* __restrict__ Dp,
+                                                       int heads, int P, int N, int G, int NG,
+                                                       const int* __restrict__ seg, float* __restrict__ state,
+                                                       float* __restrict__ y, int64_t ys) {
+  __shared__ float part[256];
+  const int sgi = blockIdx.x / heads, h = blockIdx.x - sgi * heads;
+  const int64_t row = seg[4 * sgi];
+  const int p0s = seg[4 * sgi + 2], slot = seg[4 * sgi + 3];
+  const int tid = threadIdx.x, p = tid % P, g = tid / P;
+  const int grp = h / (heads / G), inner = heads * P;
+  const float raw = ldf(proj + row * ps + dt_off + h) + dt_bias[h];
+  const float dt = raw > 20.f ? raw : log1pf(expf(raw));
+  const float dA = expf(-expf(A_log[h]) * dt);
+  const AT* xr = xbc + row * xs;
+  const float xv = ldf(xr + h * P + p), dx = dt * xv;
+  const AT* Br = xr + inner + grp * N;
+  const AT* Cr = Br + (int64_t)G * N;
+  float* st = state + ((int64_t)slot * heads + h) * N * P + p;
+  float acc = 0.f;
+  if (p0s > 0) {
+#pragma unroll 4
+    for (int nn = g; nn < N; nn += NG) {
+      const float sv = dA * st[(int64_t)nn * P] + ldf(Br + nn) * dx;
+      st[(int64_t)nn * P] = sv;
+      acc += sv * ldf(Cr + nn);
+    }
+  } else {  // first token of its sequence: the slot is written, not read
+#pragma unroll 4
+    for (int nn = g; nn < N; nn += NG) {
+      const float sv = ldf(Br + nn) * dx;
+      st[(int64_t)nn * P] = sv;
+      acc += sv * ldf(Cr + nn);
+    }
+  }
+  part[tid] = acc;
+  __syncthreads();
+  if (g == 0) {
+    float s = 0.f;
+    for (int gg = 0; gg < NG; ++gg) s += part[gg * P + p];
+    y[row * ys + h * P + p] = s + Dp[h] * xv;
   }
 }
 
@@ -937,13 +999,27 @@ int kafka_hy_scan_groups(int P, int N) {
 
 hipError_t kafka_hy_ssm_scan(int f32, const void* xbc, int64_t xs, const void* proj, int64_t ps, int dt_off,
                              const float* dt_bias, const float* A_log, const float* Dp, int heads, int P, int N, int G,
-                             const int* seg, int R, float* state, float* y, int64_t ys, hipStream_t st) {
+                             const int* seg, int R, int single, float* state, float* y, int64_t ys, hipStream_t st) {
   if (R <= 0) return hipSuccess;
+  if (single && P <= 256) {  // every segment one row
+    const int NG = std::max(1, std::min(256 / P, N));
+    DISPATCH_AT(f32, ssm_step_kernel<AT><<<R * heads, P * NG, 0, st>>>((const AT*)xbc, xs, (const AT*)proj, ps, dt_off,
+                                                                      dt_bias, A_log, Dp, heads, P, N, G, NG, seg,
+                                                                      state, y, ys));
+    return hipGetLastError();
+  }
   ScanPlan sp;
   if (!scan_plan(P, N, (int64_t)R * heads, &sp)) return hipErrorInvalidValue;
-  DISPATCH_AT(f32, ssm_scan_kernel<AT, 8, 4><<<R * heads * sp.NPS, sp.threads, sp.lds, st>>>(
-                       (const AT*)xbc, xs, (const AT*)proj, ps, dt_off, dt_bias, A_log, Dp, heads, P, N, G, sp.TN,
-                       sp.TP, sp.NPS, sp.TB, seg, state, y, ys));
+  DISPATCH_AT(f32, {
+    auto a = [&](auto k) {
+      k<<<R * heads * sp.NPS, sp.threads, sp.lds, st>>>((const AT*)xbc, xs, (const AT*)proj, ps, dt_off, dt_bias, A_log,
+                                                        Dp, heads, P, N, G, sp.TN, sp.TP, sp.NPS, seg, state, y, ys);
+    };
+    if (sp.TB == 8) a(ssm_scan_kernel<AT, 8, 4, 8>);
+    else if (sp.TB == 4) a(ssm_scan_kernel<AT, 8, 4, 4>);
+    else if (sp.TB == 2) a(ssm_scan_kernel<AT, 8, 4, 2>);
+    else a(ssm_scan_kernel<AT, 8, 4, 1>);
+  });
   return hipGetLastError();
 }
 

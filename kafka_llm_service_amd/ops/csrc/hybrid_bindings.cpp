@@ -40,7 +40,7 @@ hipError_t kafka_hy_conv_silu(int f32, const void* proj, int64_t ps, int c0, con
 int kafka_hy_scan_groups(int P, int N);
 hipError_t kafka_hy_ssm_scan(int f32, const void* xbc, int64_t xs, const void* proj, int64_t ps, int dt_off,
                              const float* dt_bias, const float* A_log, const float* Dp, int heads, int P, int N, int G,
-                             const int* seg, int R, float* state, float* y, int64_t ys, hipStream_t st);
+                             const int* seg, int R, int single, float* state, float* y, int64_t ys, hipStream_t st);
 hipError_t kafka_hy_gated_norm(int f32, const float* y, int64_t ys, const void* z, int64_t zs, const void* w, int inner,
                                int groups, float eps, void* out, int64_t os, int64_t T, hipStream_t st);
 }
@@ -332,7 +332,8 @@ void ssm_scan(at::Tensor xbc, at::Tensor proj, int64_t dt_off, at::Tensor dt_bia
   TORCH_CHECK(kafka_hy_scan_groups((int)P, (int)N) > 0, "ssm_scan: state of ", N, " x ", P, " per head is not supported");
   HY_HIP(kafka_hy_ssm_scan(f32, xbc.data_ptr(), xbc.stride(0), proj.data_ptr(), proj.stride(0), (int)dt_off,
                            dt_bias.data_ptr<float>(), A_log.data_ptr<float>(), D.data_ptr<float>(), (int)heads, (int)P,
-                           (int)N, (int)G, seg.data_ptr<int>(), (int)seg.size(0), state.data_ptr<float>(),
+                           (int)N, (int)G, seg.data_ptr<int>(), (int)seg.size(0), (int)(T == seg.size(0)),
+                           state.data_ptr<float>(),
                            y.data_ptr<float>(), y.stride(0), stream()));
 }
 

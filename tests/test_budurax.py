@@ -410,6 +410,22 @@ def test_scan_state_sizes(device, P, N):
         S = torch.exp(-torch.exp(A_log.double()) * dt)[:, None, None] * S + dt[:, None, None] * B[None, :, None] * x[:, None]
         want = (torch.einsum("hnp,n->hp", S, Cc) + x).reshape(-1)
         assert torch.allclose(y[t].cpu().double(), want, atol=1e-4, rtol=1e-4), t
+    # a step of single tokens (the decode kernel): the same sequence goes on, beside another one's first token in a
+    # slot that holds NaN
+    state = torch.cat([state, torch.full_like(state, float("nan"))])
+    xb2, pr2 = torch.randn(2, C) / 2, torch.randn(2, Hh)
+    seg, ts = _seg(device, [(1, T, 0), (1, 0, 1)])
+    y2 = torch.empty(2, inner, device=device)
+    hops.ssm_scan(xb2.to(device), pr2.to(device), 0, dt_bias.to(device), A_log.to(device), D.to(device), Hh, P, N, G,
+                  ts, seg, state, y2)
+    for r, S0 in ((0, S), (1, torch.zeros_like(S))):
+        x = xb2[r, :inner].double().view(Hh, P)
+        B, Cc = xb2[r, inner:inner + N].double(), xb2[r, inner + N:].double()
+        dt = torch.log1p(torch.exp(pr2[r].double()))
+        S1 = torch.exp(-torch.exp(A_log.double()) * dt)[:, None, None] * S0 + dt[:, None, None] * B[None, :, None] * x[:, None]
+        want = (torch.einsum("hnp,n->hp", S1, Cc) + x).reshape(-1)
+        assert torch.allclose(y2[r].cpu().double(), want, atol=1e-4, rtol=1e-4), r
+        assert torch.allclose(state[r].cpu().double(), S1, atol=1e-4, rtol=1e-4), r
 
 
 # ---- the model in the engine ---------------------------------------------------------------------------------------
