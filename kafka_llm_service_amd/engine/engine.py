@@ -231,6 +231,10 @@ class LLMEngine:
         computed from its first token."""
         from kafka_llm_service_amd.runtime import StateSlots
 
+        mode = os.environ.get("KAFKA_DECODE_GEMM", cfg.decode_gemm)
+        if mode in ("auto", "stream") and self.device.type == "cuda" and cfg.dtype == "bfloat16" and \
+                not self.model.stream:
+            self.model.enable_stream_weights()  # decode-sized steps on the weight-streaming GEMM (tiled copies)
         self.load_s = time.perf_counter() - t0
         self.eos = set(cfg.eos_token_ids or mc.eos_token_ids)
         self.fi = faults.get()

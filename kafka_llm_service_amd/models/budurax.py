@@ -35,6 +35,7 @@ from pathlib import Path
 import torch
 import torch.nn.functional as F
 
+from kafka_llm_service_amd import ops
 from kafka_llm_service_amd.ops import hybrid as hops
 
 PAGE = 16
@@ -250,11 +251,43 @@ class BuduraxLM:
         self.has_dwa = False
 
     # engine hooks shared with TransformerLM ------------------------------------------------------------------
+    STREAMED = ("qgd", "in_w", "o", "gate_up", "down")
+
+    def _streamable(self, w) -> bool:
+        return w is not None and w.dtype == torch.bfloat16 and w.is_cuda and \
+            ops.stream_plan(1, w.shape[0], w.shape[1]) is not None
+
     def stream_weight_bytes(self) -> int:
-        return 0
+        ws = [getattr(lw, n, None) for lw in self.layers for n in self.STREAMED] + [self.head]
+        return sum(w.numel() * w.element_size() for w in ws if self._streamable(w))
 
     def enable_stream_weights(self, tiled_only: bool = False) -> int:
-        return 0
+        """Wave-tiled copies of the projections (ops.tile_weight) so that decode-sized steps (<= ops.STREAM_MAX_M
+        rows) run them on the framework's weight-streaming MFMA GEMM, as the Llama path does; prefill-sized steps and
+        shapes the kernel does not take stay on hipBLASLt. bf16 only. Returns the added bytes."""
+        added = 0
+        for lw in self.layers:
+            for n in self.STREAMED:
+                w = getattr(lw, n, None)
+                if self._streamable(w):
+                    setattr(lw, n + "_t", ops.tile_weight(w))
+                    added += w.numel() * w.element_size()
+        if self._streamable(self.head):
+            self.head_t = ops.tile_weight(self.head)
+            added += self.head.numel() * self.head.element_size()
+        self.stream = added > 0
+        self.stream_max_m = ops.STREAM_MAX_M
+        return added
+
+    def _lin(self, x, w, wt=None):
+        """x @ w^T: the weight-streaming kernel for decode-sized steps when the weight has a tiled copy (its split-K
+        slabs summed to bf16 by slab_reduce), else hipBLASLt."""
+        M = x.shape[0]
+        if self.stream and wt is not None and 0 < M <= self.stream_max_m and \
+                ops.stream_plan(M, w.shape[0], w.shape[1]) is not None:
+            y = ops.linear_stream(x, wt)
+            return ops.slab_reduce(y) if ops.is_slab(y) else y
+        return F.linear(x, w)
 
     def weight_bytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in self._tensors)
@@ -425,8 +458,8 @@ class BuduraxLM:
             if lw.gate_up is not None:
                 hops.add_ln(x, y, lw.norm1b, lw.norm1b_b, eps, h2, lw.norm2, lw.norm2_b)
                 a = torch.empty(T, lw.ff, dtype=dt, device=dev)
-                hops.gelu_mul(F.linear(h2, lw.gate_up), a)
-                y = F.linear(a, lw.down)
+                hops.gelu_mul(self._lin(h2, lw.gate_up, getattr(lw, "gate_up_t", None)), a)
+                y = self._lin(a, lw.down, getattr(lw, "down_t", None))
                 nw, nb = lw.norm2b, lw.norm2b_b
             else:
                 nw, nb = lw.norm1b, lw.norm1b_b
@@ -445,13 +478,13 @@ class BuduraxLM:
         xs = x.index_select(0, inp.logit_rows)
         hf = torch.empty(xs.shape[0], d, dtype=dt, device=dev)
         hops.ln_shift(xs, self.final_norm, self.final_norm_b, eps, hf)
-        return F.linear(hf, self.head).float()[:, :cfg.vocab_size]
+        return self._lin(hf, self.head, getattr(self, "head_t", None)).float()[:, :cfg.vocab_size]
 
     def _latent_attention(self, i: int, lw, h, inp, m: SegMeta, pages: list) -> torch.Tensor:
         mm = lw.m
         H, D, rd, vd, R = (int(mm[k]) for k in ("heads", "dim", "rot_dim", "vdim", "kv_rank"))
         T, dt, dev = h.shape[0], self.dtype, self.device
-        qgd = F.linear(h, lw.qgd)  # [q heads (dim | rot) | output gate | latent, shared rotary key]
+        qgd = self._lin(h, lw.qgd, getattr(lw, "qgd_t", None))  # [q heads (dim | rot) | output gate | latent, shared rotary key]
         src = i if lw.kv_from is None else int(lw.kv_from)
         cache, cache_t = pages[src], self.pages_t[src]
         q_rot = torch.empty(T, H, rd, dtype=dt, device=dev)
@@ -465,21 +498,21 @@ class BuduraxLM:
         a = torch.bmm(o_lat, lw.uv_ht)                                            # [H, T, vdim]
         ao = torch.empty(T, H * vd, dtype=dt, device=dev)
         hops.sigmoid_mul(a, qgd[:, lw.g_off:lw.g_off + H * vd], ao)
-        return F.linear(ao, lw.o)
+        return self._lin(ao, lw.o, getattr(lw, "o_t", None))
 
     def _mamba2(self, i: int, lw, h, m: SegMeta, state: RecurrentState) -> torch.Tensor:
         mm = lw.m
         Hh, P, N, G = (int(mm[k]) for k in ("heads", "vdim", "state", "groups"))
         inner, C = Hh * P, Hh * P + 2 * G * N
         T, dt, dev = h.shape[0], self.dtype, self.device
-        proj = F.linear(h, lw.in_w)  # [z | x | B | C | dt]
+        proj = self._lin(h, lw.in_w, getattr(lw, "in_w_t", None))  # [z | x | B | C | dt]
         xbc = torch.empty(T, C, dtype=dt, device=dev)
         hops.conv_silu(proj, inner, lw.conv, lw.conv_b, m.tok_seg, m.seg, state.conv[i], xbc)
         y = torch.empty(T, inner, dtype=torch.float32, device=dev)
         hops.ssm_scan(xbc, proj, inner + C, lw.dt_bias, lw.A_log, lw.D, Hh, P, N, G, m.tok_seg, m.seg, state.ssm[i], y)
         yn = torch.empty(T, inner, dtype=dt, device=dev)
         hops.gated_norm(y, proj, lw.mnorm, int(mm["norm_groups"]), self.cfg.norm_eps, yn)
-        return F.linear(yn, lw.o)
+        return self._lin(yn, lw.o, getattr(lw, "o_t", None))
 
 
 def load_checkpoint(model: BuduraxLM, path: str | Path) -> BuduraxLM:

@@ -84,9 +84,12 @@ class ServerConfig:
 
 
 def _engine_kwargs(e) -> dict[str, Any]:
-    """Engine options from the environment: KAFKA_KV_DTYPE (bf16 | fp8 KV cache), KAFKA_GRAPHS=1 (hipGraph decode
-    steps), KAFKA_MAX_NUM_SEQS, KAFKA_MAX_BATCHED_TOKENS."""
+    """Engine options from the environment: KAFKA_KV_DTYPE (bf16 | fp8 KV cache), KAFKA_DTYPE (bfloat16 | float32
+    activations, the latter for the model families built for it), KAFKA_GRAPHS=1 (hipGraph decode steps),
+    KAFKA_MAX_NUM_SEQS, KAFKA_MAX_BATCHED_TOKENS."""
     kw: dict[str, Any] = {}
+    if e.get("KAFKA_DTYPE"):
+        kw["dtype"] = e["KAFKA_DTYPE"]
     if e.get("KAFKA_KV_DTYPE"):
         kw["kv_dtype"] = e["KAFKA_KV_DTYPE"]
     if e.get("KAFKA_GRAPHS") in ("0", "1"):  # unset: the engine's default (on for TP > 1)

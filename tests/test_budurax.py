@@ -340,6 +340,25 @@ def test_matrix_core_attention_in_the_engine():
     assert eng.kvm.num_free() == 40
 
 
+@pytest.mark.gpu
+def test_streamed_projections():
+    """Decode-sized steps run the projections on the weight-streaming GEMM when their shapes fit it (width 256 here):
+    single tokens and a 100-token portion (streamed) against the plain model, and the same steps with streaming off."""
+    ff = {"kind": "dense", "ff": 512}
+    cfg = {"architecture": "Budurax", "vocab": 320, "width": 256, "norm": {"eps": 1e-5}, "token_side": {"dim": 8},
+           "layers": [{"type": "latent_attention", "mixer": _attn(4, 32, 32, 32, 64, 64), "mlp": ff},
+                      {"type": "mamba2", "mixer": _mamba(8, 32, 16, 2, 2, 4), "mlp": ff}]}
+    b = Bench(cfg, seed=12)
+    t = toks(140, 320, 3)
+    outs = []
+    for mode in ("stream", "blas"):
+        eng = b.engine("cuda:0", "bfloat16", decode_gemm=mode)
+        assert eng.model.stream == (mode == "stream")
+        outs.append(feed_all(eng, "r", t, [100, 1]))
+        assert rel_err(outs[-1], b.oracle(t)) < TOL["bfloat16"]
+    assert rel_err(outs[0], outs[1].float().cpu()) < TOL["bfloat16"]
+
+
 @pytest.mark.parametrize("device", DEVICES)
 def test_conv_and_scan_portions(device):
     """Convolution tail and state-space state carried over portions of 1, 2, 3 and 7 rows, with another sequence's run
