@@ -854,7 +854,8 @@ class ModelRunner:
             n_bt = nbt * h.bt_w
             sm = SegMeta(T, h.n_seg, d32[n_bt + T:n_bt + T + 4 * h.n_seg].view(h.n_seg, 4), d32[n_bt:n_bt + T],
                          d32[:n_bt].view(nbt, h.bt_w),
-                         {tt: d32[o:o + 4 * n].view(n, 4) for tt, o, n in h.tiles})
+                         {tt: d32[o:o + 4 * n].view(n, 4) for tt, o, n in h.tiles},
+                         seg_host=np.asarray(h.i32[n_bt + T:n_bt + T + 4 * h.n_seg]).reshape(h.n_seg, 4))
             if h.n_late:
                 L, n = h.late_off, h.n_late
                 t_tokens.index_copy_(0, d64[L:L + n], self.tok_buf.index_select(0, d64[L + n:L + 2 * n]))

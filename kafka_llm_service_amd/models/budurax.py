@@ -213,6 +213,8 @@ class SegMeta:
     block_tables: torch.Tensor
     # attention tiles per tile size in tokens: int32 [n, 4] = (first row, tokens, run, 0), each within one run
     tiles: dict = field(default_factory=dict)
+    seg_host: object = None   # numpy copy of ``seg`` (the plan's host side), for launch-shape decisions
+    cache: dict = field(default_factory=dict)   # per-step device tables derived from seg_host (chunk plans)
 
 
 @dataclass
@@ -500,6 +502,20 @@ class BuduraxLM:
         hops.sigmoid_mul(a, qgd[:, lw.g_off:lw.g_off + H * vd], ao)
         return self._lin(ao, lw.o, getattr(lw, "o_t", None))
 
+    def _chunk_plan(self, m: SegMeta, heads: int):
+        """Device chunk tables of this step for layers of ``heads`` heads (built once per step), None = plain scan."""
+        key = ("chunks", heads)
+        if key not in m.cache:
+            p = hops.scan_chunks(m.seg_host, heads)
+            if p is not None:
+                fresh, cont, cs, mx = p
+                up = torch.from_numpy(__import__("numpy").concatenate([fresh.reshape(-1), cont.reshape(-1),
+                                                                       cs.reshape(-1)])).to(self.device)
+                a, b = fresh.size, fresh.size + cont.size
+                p = (up[:a].view(-1, 4), up[a:b].view(-1, 4), up[b:].view(-1, 4), mx)
+            m.cache[key] = p
+        return m.cache[key]
+
     def _mamba2(self, i: int, lw, h, m: SegMeta, state: RecurrentState) -> torch.Tensor:
         mm = lw.m
         Hh, P, N, G = (int(mm[k]) for k in ("heads", "vdim", "state", "groups"))
@@ -509,7 +525,12 @@ class BuduraxLM:
         xbc = torch.empty(T, C, dtype=dt, device=dev)
         hops.conv_silu(proj, inner, lw.conv, lw.conv_b, m.tok_seg, m.seg, state.conv[i], xbc)
         y = torch.empty(T, inner, dtype=torch.float32, device=dev)
-        hops.ssm_scan(xbc, proj, inner + C, lw.dt_bias, lw.A_log, lw.D, Hh, P, N, G, m.tok_seg, m.seg, state.ssm[i], y)
+        plan = self._chunk_plan(m, Hh) if dev.type == "cuda" else None
+        if plan is not None:  # long prompt portions, few sequences: chunk-parallel scan
+            hops.ssm_scan_chunked(xbc, proj, inner + C, lw.dt_bias, lw.A_log, lw.D, Hh, P, N, G, plan, state.ssm[i], y)
+        else:
+            hops.ssm_scan(xbc, proj, inner + C, lw.dt_bias, lw.A_log, lw.D, Hh, P, N, G, m.tok_seg, m.seg,
+                          state.ssm[i], y)
         yn = torch.empty(T, inner, dtype=dt, device=dev)
         hops.gated_norm(y, proj, lw.mnorm, int(mm["norm_groups"]), self.cfg.norm_eps, yn)
         return self._lin(yn, lw.o, getattr(lw, "o_t", None))

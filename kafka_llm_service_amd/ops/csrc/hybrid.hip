@@ -782,6 +782,47 @@ __global__ __launch_bounds__(256) void ssm_step_kernel(const AT* __restrict__ xb
   }
 }
 
+// Chunk-parallel scan, middle pass. A long segment is cut into chunks that are first scanned independently from a
+// zero state (ssm_scan over the chunk table `vseg`); here the chunks' entry states are rebuilt in order,
+//   S_in[0] = the sequence's state (zero at position 0),  S_in[c + 1] = D_c S_in[c] + S_loc[c],
+// with D_c = exp(-exp(A_log) sum of the chunk's step sizes), S_in[c] replaces S_loc[c] in the chunk's scratch slot (the
+// second scan starts from it) and the value after the last chunk is the sequence's new state. One workgroup per
+// (segment, head); cs[s] = (first chunk, chunks, first position, state slot).
+template <typename AT>
+__global__ __launch_bounds__(256) void ssm_combine_kernel(const AT* __restrict__ proj, int64_t ps, int dt_off,
+                                                          const float* __restrict__ dt_bias,
+                                                          const float* __restrict__ A_log, int heads, int NP_,
+                                                          const int* __restrict__ vseg, const int* __restrict__ cs,
+                                                          float* __restrict__ tmp, float* __restrict__ state) {
+  __shared__ float red[4];
+  __shared__ float D[256];
+  const int sgi = blockIdx.x / heads, h = blockIdx.x - sgi * heads;
+  const int c0 = cs[4 * sgi], nch = cs[4 * sgi + 1], p0 = cs[4 * sgi + 2], slot = cs[4 * sgi + 3];
+  const float A = -expf(A_log[h]), bias = dt_bias[h];
+  for (int c = 0; c < nch; ++c) {
+    const int q0 = vseg[4 * (c0 + c)], n = vseg[4 * (c0 + c) + 1];
+    float sdt = 0.f;
+    for (int t = threadIdx.x; t < n; t += 256) {
+      const float raw = ldf(proj + (int64_t)(q0 + t) * ps + dt_off + h) + bias;
+      sdt += raw > 20.f ? raw : log1pf(expf(raw));
+    }
+    sdt = block_sum<256>(sdt, red);
+    if (threadIdx.x == 0) D[c] = expf(A * sdt);
+  }
+  __syncthreads();
+  float* st = state + ((int64_t)slot * heads + h) * NP_;
+  for (int e = threadIdx.x; e < NP_; e += 256) {
+    float sv = p0 > 0 ? st[e] : 0.f;
+    for (int c = 0; c < nch; ++c) {
+      float* tp = tmp + ((int64_t)vseg[4 * (c0 + c) + 3] * heads + h) * NP_ + e;
+      const float loc = *tp;
+      *tp = sv;
+      sv = D[c] * sv + loc;
+    }
+    st[e] = sv;
+  }
+}
+
 template <typename AT>
 __global__ __launch_bounds__(NT) void gated_norm_kernel(const float* __restrict__ y, int64_t ys, const AT* __restrict__ z,
                                                         int64_t zs, const AT* __restrict__ w, int gs, float eps,
@@ -1020,6 +1061,15 @@ hipError_t kafka_hy_ssm_scan(int f32, const void* xbc, int64_t xs, const void* p
     else if (sp.TB == 2) a(ssm_scan_kernel<AT, 8, 4, 2>);
     else a(ssm_scan_kernel<AT, 8, 4, 1>);
   });
+  return hipGetLastError();
+}
+
+hipError_t kafka_hy_ssm_combine(int f32, const void* proj, int64_t ps, int dt_off, const float* dt_bias,
+                                const float* A_log, int heads, int NP_, const int* vseg, const int* cs, int S,
+                                float* tmp, float* state, hipStream_t st) {
+  if (S <= 0) return hipSuccess;
+  DISPATCH_AT(f32, ssm_combine_kernel<AT><<<S * heads, 256, 0, st>>>((const AT*)proj, ps, dt_off, dt_bias, A_log, heads,
+                                                                    NP_, vseg, cs, tmp, state));
   return hipGetLastError();
 }
 

@@ -41,6 +41,9 @@ int kafka_hy_scan_groups(int P, int N);
 hipError_t kafka_hy_ssm_scan(int f32, const void* xbc, int64_t xs, const void* proj, int64_t ps, int dt_off,
                              const float* dt_bias, const float* A_log, const float* Dp, int heads, int P, int N, int G,
                              const int* seg, int R, int single, float* state, float* y, int64_t ys, hipStream_t st);
+hipError_t kafka_hy_ssm_combine(int f32, const void* proj, int64_t ps, int dt_off, const float* dt_bias,
+                                const float* A_log, int heads, int NP_, const int* vseg, const int* cs, int S,
+                                float* tmp, float* state, hipStream_t st);
 hipError_t kafka_hy_gated_norm(int f32, const float* y, int64_t ys, const void* z, int64_t zs, const void* w, int inner,
                                int groups, float eps, void* out, int64_t os, int64_t T, hipStream_t st);
 }
@@ -337,6 +340,30 @@ void ssm_scan(at::Tensor xbc, at::Tensor proj, int64_t dt_off, at::Tensor dt_bia
                            y.data_ptr<float>(), y.stride(0), stream()));
 }
 
+// vseg int32 [V, 4] chunk table (first row, rows, -, scratch slot); cs int32 [S, 4] = (first chunk, chunks, first
+// position, state slot); at most 256 chunks per segment
+void ssm_combine(at::Tensor proj, int64_t dt_off, at::Tensor dt_bias, at::Tensor A_log, int64_t heads, at::Tensor vseg,
+                 at::Tensor cs, int64_t max_chunks, at::Tensor tmp, at::Tensor state) {
+  rows2d(proj, "proj");
+  const int f32 = act_f32(proj);
+  TORCH_CHECK(dt_off >= 0 && dt_off + heads <= proj.size(1) && max_chunks >= 1 && max_chunks <= 256,
+              "ssm_combine: sizes (at most 256 chunks per segment)");
+  for (const at::Tensor* t : {&dt_bias, &A_log})
+    TORCH_CHECK(t->is_cuda() && t->scalar_type() == at::kFloat && t->is_contiguous() && t->numel() == heads,
+                "ssm_combine: dt_bias / A_log fp32 [heads]");
+  for (const at::Tensor* t : {&vseg, &cs})
+    TORCH_CHECK(t->is_cuda() && t->scalar_type() == at::kInt && t->is_contiguous() && t->dim() == 2 && t->size(1) == 4,
+                "ssm_combine: int32 [n, 4] tables");
+  TORCH_CHECK(tmp.is_cuda() && tmp.scalar_type() == at::kFloat && tmp.is_contiguous() && tmp.dim() == 4 &&
+                  state.is_cuda() && state.scalar_type() == at::kFloat && state.is_contiguous() && state.dim() == 4 &&
+                  tmp.size(0) >= vseg.size(0) && tmp.size(1) == heads && state.size(1) == heads &&
+                  tmp.size(2) == state.size(2) && tmp.size(3) == state.size(3), "ssm_combine: state tensors");
+  HY_HIP(kafka_hy_ssm_combine(f32, proj.data_ptr(), proj.stride(0), (int)dt_off, dt_bias.data_ptr<float>(),
+                              A_log.data_ptr<float>(), (int)heads, (int)(state.size(2) * state.size(3)),
+                              vseg.data_ptr<int>(), cs.data_ptr<int>(), (int)cs.size(0), tmp.data_ptr<float>(),
+                              state.data_ptr<float>(), stream()));
+}
+
 void gated_norm(at::Tensor y, at::Tensor proj, at::Tensor w, int64_t groups, double eps, at::Tensor out) {
   rows2d(y, "y"); rows2d(proj, "proj"); rows2d(out, "out");
   const int f32 = act_f32(proj);
@@ -372,6 +399,7 @@ void kafka_bind_hybrid(pybind11::module_& m) {
   m.def("hy_latent_attn", &latent_attn);
   m.def("hy_conv_silu", &conv_silu);
   m.def("hy_ssm_scan", &ssm_scan);
+  m.def("hy_ssm_combine", &ssm_combine);
   m.def("hy_gated_norm", &gated_norm);
   m.def("hy_scan_groups", [](int P, int N) { return kafka_hy_scan_groups(P, N); });
 }

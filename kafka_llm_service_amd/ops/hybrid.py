@@ -146,6 +146,48 @@ def ssm_scan(xbc, proj, dt_off: int, dt_bias, A_log, D, heads, P, N, G, tok_seg,
         ref.ssm_scan(xbc, proj, dt_off, dt_bias, A_log, D, heads, P, N, G, tok_seg, seg, state, y)
 
 
+SCAN_CHUNK = 256        # tokens per chunk of the chunk-parallel scan
+SCAN_CHUNK_MIN = 512    # a step is scanned in chunks when its longest segment has at least this many rows ...
+SCAN_CHUNK_WORK = 2048  # ... and it has fewer (segment, head) pairs than this (else the plain scan fills the GPU)
+
+
+def scan_chunks(seg_host, heads: int):
+    """Chunk tables of a step for the chunk-parallel scan, or None when the plain scan is the better fit:
+    (vseg_fresh, vseg_cont, cs, max chunks) as numpy int32 - every segment cut into chunks of SCAN_CHUNK rows, chunk c
+    of the step using scratch slot c; vseg_fresh starts every chunk from zero, vseg_cont from its scratch slot."""
+    import numpy as np
+
+    if seg_host is None or len(seg_host) == 0:
+        return None
+    n_max = int(seg_host[:, 1].max())
+    if n_max < SCAN_CHUNK_MIN or len(seg_host) * heads >= SCAN_CHUNK_WORK or n_max > 256 * SCAN_CHUNK:
+        return None
+    vs, cs = [], []
+    for q0, n, p0, slot in seg_host.tolist():
+        first = len(vs)
+        for a in range(0, n, SCAN_CHUNK):
+            vs.append((q0 + a, min(SCAN_CHUNK, n - a), 0, len(vs)))
+        cs.append((first, len(vs) - first, p0, slot))
+    fresh = np.asarray(vs, dtype=np.int32)
+    cont = fresh.copy()
+    cont[:, 2] = 1
+    return fresh, cont, np.asarray(cs, dtype=np.int32), max(c[1] for c in cs)
+
+
+def ssm_scan_chunked(xbc, proj, dt_off: int, dt_bias, A_log, D, heads, P, N, G, plan, state, y) -> None:
+    """The recurrence of ``ssm_scan`` in three launches that expose more parallelism for long segments: every chunk
+    scanned from a zero state, the chunks' entry states rebuilt in order (and the sequence's state advanced), every
+    chunk scanned again from its entry state. ``plan``: device tensors (vseg_fresh, vseg_cont, cs) + max chunks from
+    ``scan_chunks``. Twice the arithmetic of the plain scan over (chunks) times the workgroups; the result differs
+    from the token-by-token order only by fp32 rounding (the entry states are re-associated)."""
+    fresh, cont, cs, max_chunks = plan
+    tmp = torch.empty(fresh.shape[0], heads, N, P, dtype=torch.float32, device=xbc.device)
+    e = ext()
+    e.hy_ssm_scan(xbc, proj, int(dt_off), dt_bias, A_log, D, int(heads), int(P), int(N), int(G), fresh, tmp, y)
+    e.hy_ssm_combine(proj, int(dt_off), dt_bias, A_log, int(heads), fresh, cs, int(max_chunks), tmp, state)
+    e.hy_ssm_scan(xbc, proj, int(dt_off), dt_bias, A_log, D, int(heads), int(P), int(N), int(G), cont, tmp, y)
+
+
 def gated_norm(y, proj, w, groups: int, eps, out) -> None:
     """out = group_rms_norm(y * silu(proj[:, :inner])) * w, the norm over ``groups`` equal parts of a row."""
     if _gpu(y):

@@ -341,6 +341,52 @@ def test_matrix_core_attention_in_the_engine():
 
 
 @pytest.mark.gpu
+def test_chunk_parallel_scan():
+    """Long segments scanned in chunks (zero-state scan, ordered rebuild of the entry states, second scan) against the
+    token-by-token reference: a fresh 700-row segment, a 3-row one and a 600-row one that continue stored states."""
+    from kafka_llm_service_amd.ops import hybrid_reference as href
+
+    device = "cuda:0"
+    torch.manual_seed(6)
+    Hh, P, N, G = 6, 24, 40, 2
+    inner, C = Hh * P, Hh * P + 2 * G * N
+    runs = [(700, 0, 1), (3, 5, 0), (600, 40, 2)]
+    T = sum(r[0] for r in runs)
+    xbc, proj = torch.randn(T, C) / 2, torch.randn(T, inner + C + Hh)
+    dt_bias, A_log, D = torch.randn(Hh) / 2 - 2.0, torch.rand(Hh), torch.randn(Hh)
+    state0 = torch.randn(3, Hh, N, P)
+    seg, ts = _seg("cpu", runs)
+    want_state, want_y = state0.clone(), torch.empty(T, inner)
+    href.ssm_scan(xbc, proj, inner + C, dt_bias, A_log, D, Hh, P, N, G, ts, seg, want_state, want_y)
+    plan = hops.scan_chunks(seg.numpy(), Hh)
+    assert plan is not None and plan[3] == 3 and plan[0].shape[0] == 3 + 1 + 3
+    dplan = tuple(torch.from_numpy(a).to(device) for a in plan[:3]) + (plan[3],)
+    state, y = state0.clone().to(device), torch.empty(T, inner, device=device)
+    hops.ssm_scan_chunked(xbc.to(device), proj.to(device), inner + C, dt_bias.to(device), A_log.to(device),
+                          D.to(device), Hh, P, N, G, dplan, state, y)
+    assert torch.allclose(y.cpu(), want_y, atol=2e-4, rtol=2e-4)
+    assert torch.allclose(state.cpu(), want_state, atol=2e-4, rtol=2e-4)
+    assert hops.scan_chunks(_seg("cpu", [(100, 0, 0)])[0].numpy(), Hh) is None      # short: plain scan
+    assert hops.scan_chunks(_seg("cpu", [(600, 0, 0)])[0].numpy(), 4096) is None    # enough workgroups already
+
+
+@pytest.mark.gpu
+def test_long_prompt_in_the_engine():
+    """A 900-token prompt in one step, and in portions of 600 + 300 (chunk-parallel scan in both), beside a short
+    request, against the plain model (fp32)."""
+    b = Bench(cfg_a(), seed=13)
+    t, u = toks(900, 211, 4), toks(30, 211, 5)
+    eng = b.engine("cuda:0", "float32", blocks=80)
+    assert rel_err(feed_all(eng, "w", t, [900]), b.oracle(t)) < TOL["float32"]
+    got = [eng.feed([("t", t[:600], list(range(600))), ("u", u[:29], list(range(29)))])]
+    got.append(eng.feed([("u", u[29:], [0]), ("t", t[600:], list(range(300)))], ["t", "u"]))
+    got_t = torch.cat([got[0][:600], got[1][1:]])
+    got_u = torch.cat([got[0][600:], got[1][:1]])
+    assert rel_err(got_t, b.oracle(t)) < TOL["float32"]
+    assert rel_err(got_u, b.oracle(u)) < TOL["float32"]
+
+
+@pytest.mark.gpu
 def test_streamed_projections():
     """Decode-sized steps run the projections on the weight-streaming GEMM when their shapes fit it (width 256 here):
     single tokens and a 100-token portion (streamed) against the plain model, and the same steps with streaming off."""
