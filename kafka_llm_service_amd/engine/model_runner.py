@@ -856,6 +856,7 @@ class ModelRunner:
                          d32[:n_bt].view(nbt, h.bt_w),
                          {tt: d32[o:o + 4 * n].view(n, 4) for tt, o, n in h.tiles},
                          seg_host=np.asarray(h.i32[n_bt + T:n_bt + T + 4 * h.n_seg]).reshape(h.n_seg, 4))
+            sm.max_keys = int((sm.seg_host[:, 1] + sm.seg_host[:, 2]).max()) if h.n_seg else 0
             if h.n_late:
                 L, n = h.late_off, h.n_late
                 t_tokens.index_copy_(0, d64[L:L + n], self.tok_buf.index_select(0, d64[L + n:L + 2 * n]))

@@ -214,6 +214,7 @@ class SegMeta:
     # attention tiles per tile size in tokens: int32 [n, 4] = (first row, tokens, run, 0), each within one run
     tiles: dict = field(default_factory=dict)
     seg_host: object = None   # numpy copy of ``seg`` (the plan's host side), for launch-shape decisions
+    max_keys: int = 0         # longest context of the step (first position + rows over the runs)
     cache: dict = field(default_factory=dict)   # per-step device tables derived from seg_host (chunk plans)
 
 
@@ -496,7 +497,7 @@ class BuduraxLM:
         q_lat = torch.bmm(q_u, lw.uk_h)                                           # [H, T, R]
         o_lat = torch.empty(H, T, R, dtype=dt, device=dev)
         hops.latent_attn(q_lat, q_rot, cache, m.block_tables, m.tok_seg, m.seg, inp.positions, lw.scale, o_lat,
-                         cache_t, m.tiles.get(hops.tile_tokens(H)))
+                         cache_t, m.tiles.get(hops.tile_tokens(H)), m.max_keys)
         a = torch.bmm(o_lat, lw.uv_ht)                                            # [H, T, vdim]
         ao = torch.empty(T, H * vd, dtype=dt, device=dev)
         hops.sigmoid_mul(a, qgd[:, lw.g_off:lw.g_off + H * vd], ao)

@@ -363,7 +363,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const bf16* __restrict__ q_lat, int64_t ql_h, int64_t ql_t, const bf16* __restrict__ q_rot, int64_t qr_t,
     int64_t qr_h, const bf16* __restrict__ cache, const bf16* __restrict__ cache_t, int R, int rd,
     const int* __restrict__ bt, int bt_stride, const int* __restrict__ items, const int64_t* __restrict__ positions,
-    float scale_log2e, bf16* __restrict__ out, int64_t o_h, int64_t o_t, int H) {
+    float scale_log2e, bf16* __restrict__ out, int64_t o_h, int64_t o_t, int H, float* __restrict__ po,
+    float* __restrict__ pml, int T) {
+  // gridDim.z > 1: the tile's key blocks are dealt to gridDim.z workgroups in contiguous ranges; each leaves its
+  // unnormalised accumulators in po [z][H][T][R] and (row maximum, row sum) in pml [z][H][T][2] for latent_merge
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int Dk = R + rd, nks = Dk >> 4, qstride = Dk + 8;
   bf16* Qs = reinterpret_cast<bf16*>(smem);                 // [32][Dk + 8]
@@ -423,8 +426,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     for (int ks = 0; ks < NKSC; ++ks)
       if (ks < nks) kf[ks] = load_bf16x8(krow + 16 * ks);
   };
-  if (32 * w <= maxpos) fetch_keys(0);
-  for (int kb = 0; kb < nblocks; ++kb) {
+  const int nsplit = gridDim.z;
+  const int bps = (nblocks + nsplit - 1) / nsplit;
+  const int kb0 = blockIdx.z * bps, kb1 = min(nblocks, kb0 + bps);
+  if (kb0 < kb1 && kb0 * 128 + 32 * w <= maxpos) fetch_keys(kb0);
+  for (int kb = kb0; kb < kb1; ++kb) {
     // ---- scores of this wave's 32 keys
     const int key = kb * 128 + 32 * w + lr;
     f32x16 S;
@@ -436,7 +442,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       for (int ks = 0; ks < NKSC; ++ks)
         if (ks < nks) S = mfma32(load_bf16x8(qrow + 16 * ks), kf[ks], S);
     }
-    if (kb + 1 < nblocks && (kb + 1) * 128 + 32 * w <= maxpos) fetch_keys(kb + 1);
+    if (kb + 1 < kb1 && (kb + 1) * 128 + 32 * w <= maxpos) fetch_keys(kb + 1);
     float s[16], mx[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
@@ -456,8 +462,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     for (int i = 0; i < 16; ++i) {
       const int r = (i & 3) + 8 * (i >> 2) + 4 * lh;
       const float mn = fmaxf(fmaxf(m[i], fmaxf(mloc[r], mloc[32 + r])), fmaxf(mloc[64 + r], mloc[96 + r]));
-      corr[i] = fast_exp2(m[i] - mn);  // first block: m = -inf, mn finite (key 0 is visible to every row) -> 0
-      const float p = fast_exp2(s[i] - mn);
+      // first block: m = -inf -> corr 0. A later split's range may start past a row's position: then mn is still
+      // -inf and the row stays empty (the guards keep inf - inf out)
+      corr[i] = mn == -INFINITY ? 0.f : fast_exp2(m[i] - mn);
+      const float p = mn == -INFINITY ? 0.f : fast_exp2(s[i] - mn);
       lsum[i] = lsum[i] * corr[i] + p;
       m[i] = mn;
       Ps[r * 136 + 32 * w + lr] = (bf16)p;
@@ -510,13 +518,50 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   for (int i = 0; i < 16; ++i) {
     const int r = (i & 3) + 8 * (i >> 2) + 4 * lh;
     if (r >= nrows) continue;
-    const float inv = 1.0f / (mloc[r] + mloc[32 + r] + mloc[64 + r] + mloc[96 + r]);
+    const float l = mloc[r] + mloc[32 + r] + mloc[64 + r] + mloc[96 + r];
     const int64_t t = t0 + r / hpr, h = h0 + r % hpr;
+    if (nsplit == 1) {
+      const float inv = 1.0f / l;
 #pragma unroll
-    for (int tw = 0; tw < TW; ++tw) {
-      const int ct = w * TW + tw;
-      if (ct * 32 < R) out[h * o_h + t * o_t + ct * 32 + lr] = (bf16)(O[tw][i] * inv);
+      for (int tw = 0; tw < TW; ++tw) {
+        const int ct = w * TW + tw;
+        if (ct * 32 < R) out[h * o_h + t * o_t + ct * 32 + lr] = (bf16)(O[tw][i] * inv);
+      }
+    } else {
+      const int64_t row = ((int64_t)blockIdx.z * H + h) * T + t;
+      if (w == 0 && lr == 0) {
+        pml[2 * row] = m[i];
+        pml[2 * row + 1] = l;
+      }
+#pragma unroll
+      for (int tw = 0; tw < TW; ++tw) {
+        const int ct = w * TW + tw;
+        if (ct * 32 < R) po[row * R + ct * 32 + lr] = O[tw][i];
+      }
     }
+  }
+}
+
+// out[h][t] = sum_z 2^(m_z - m) O_z / sum_z 2^(m_z - m) l_z over the key-range splits of latent_attn_mfma_kernel
+__global__ void latent_merge_kernel(const float* __restrict__ po, const float* __restrict__ pml, int nsplit, int H,
+                                    int T, int R, bf16* __restrict__ out, int64_t o_h, int64_t o_t) {
+  const int64_t ht = blockIdx.x;  // h * T + t
+  const int h = (int)(ht / T), t = (int)(ht - (int64_t)h * T);
+  float mx = -INFINITY;
+  for (int z = 0; z < nsplit; ++z) mx = fmaxf(mx, pml[2 * ((int64_t)z * H * T + ht)]);
+  float den = 0.f;
+  for (int z = 0; z < nsplit; ++z) {
+    const float mz = pml[2 * ((int64_t)z * H * T + ht)];
+    if (mz != -INFINITY) den += fast_exp2(mz - mx) * pml[2 * ((int64_t)z * H * T + ht) + 1];
+  }
+  const float inv = 1.0f / den;
+  for (int d = threadIdx.x; d < R; d += blockDim.x) {
+    float a = 0.f;
+    for (int z = 0; z < nsplit; ++z) {
+      const float mz = pml[2 * ((int64_t)z * H * T + ht)];
+      if (mz != -INFINITY) a += fast_exp2(mz - mx) * po[((int64_t)z * H * T + ht) * R + d];
+    }
+    out[(int64_t)h * o_h + (int64_t)t * o_t + d] = (bf16)(a * inv);
   }
 }
 
@@ -971,17 +1016,19 @@ hipError_t kafka_hy_latent_attn_mfma(const void* q_lat, int64_t ql_h, int64_t ql
                                      int64_t qr_h, const void* cache, const void* cache_t, int R, int rd,
                                      const int* bt, int bt_stride, const int* items, int n_items,
                                      const int64_t* positions, float scale, void* out, int64_t o_h, int64_t o_t, int H,
-                                     hipStream_t st) {
+                                     int nsplit, float* po, float* pml, int T, hipStream_t st) {
   if (n_items <= 0) return hipSuccess;
+  if (nsplit < 1 || nsplit > 64 || (nsplit > 1 && (po == nullptr || pml == nullptr))) return hipErrorInvalidValue;
   if (!kafka_hy_latent_mfma_ok(16, R, rd)) return hipErrorInvalidValue;
   const int Dk = R + rd;
   const size_t lds = (size_t)32 * (Dk + 8) * 2 + 32 * 136 * 2 + 128 * 4 + 32 * 4 + MFMA_PG * 4;
-  const dim3 grid((unsigned)n_items, (unsigned)((H + 31) / 32));
+  const dim3 grid((unsigned)n_items, (unsigned)((H + 31) / 32), (unsigned)nsplit);
   const float sl = scale * 1.4426950408889634f;
   const int tw = (R / 32 + 3) / 4;
   auto a = [&](auto k) {
     k<<<grid, 256, lds, st>>>((const bf16*)q_lat, ql_h, ql_t, (const bf16*)q_rot, qr_t, qr_h, (const bf16*)cache,
-                              (const bf16*)cache_t, R, rd, bt, bt_stride, items, positions, sl, (bf16*)out, o_h, o_t, H);
+                              (const bf16*)cache_t, R, rd, bt, bt_stride, items, positions, sl, (bf16*)out, o_h, o_t, H,
+                              po, pml, T);
   };
   const int nks = Dk / 16;
   if (tw == 1 && nks <= 12) a(latent_attn_mfma_kernel<1, 12>);
@@ -991,6 +1038,8 @@ hipError_t kafka_hy_latent_attn_mfma(const void* q_lat, int64_t ql_h, int64_t ql
   else if (tw == 3) a(latent_attn_mfma_kernel<3, 40>);
   else if (nks <= 36) a(latent_attn_mfma_kernel<4, 36>);
   else a(latent_attn_mfma_kernel<4, 40>);
+  if (nsplit > 1)
+    latent_merge_kernel<<<(unsigned)((int64_t)H * T), 128, 0, st>>>(po, pml, nsplit, H, T, R, (bf16*)out, o_h, o_t);
   return hipGetLastError();
 }
 

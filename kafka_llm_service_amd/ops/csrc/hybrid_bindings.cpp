@@ -26,7 +26,7 @@ hipError_t kafka_hy_latent_attn_mfma(const void* q_lat, int64_t ql_h, int64_t ql
                                      int64_t qr_h, const void* cache, const void* cache_t, int R, int rd,
                                      const int* bt, int bt_stride, const int* items, int n_items,
                                      const int64_t* positions, float scale, void* out, int64_t o_h, int64_t o_t, int H,
-                                     hipStream_t st);
+                                     int nsplit, float* po, float* pml, int T, hipStream_t st);
 hipError_t kafka_hy_sigmoid_mul(int f32, const void* a, int64_t a_h, int64_t a_t, const void* g, int64_t gs, void* out,
                                 int64_t T, int H, int vd, hipStream_t st);
 int kafka_hy_latent_attn_max_dk();
@@ -267,7 +267,8 @@ void latent_attn(at::Tensor q_lat, at::Tensor q_rot, at::Tensor cache, at::Tenso
 // the matrix-core kernel: items int32 [n, 4] = (first row, tokens, segment, 0), each at most 32 (token, head) rows of
 // one segment (or one token, whose heads go 32 at a time over grid.y)
 void latent_attn_mfma(at::Tensor q_lat, at::Tensor q_rot, at::Tensor cache, at::Tensor cache_t, at::Tensor bt,
-                      at::Tensor items, int64_t tile_tokens, at::Tensor positions, double scale, at::Tensor out) {
+                      at::Tensor items, int64_t tile_tokens, at::Tensor positions, double scale, at::Tensor out,
+                      int64_t nsplit, OptT po, OptT pml) {
   for (const at::Tensor* t : {&q_lat, &q_rot, &cache, &cache_t, &out})
     TORCH_CHECK(t->is_cuda() && t->scalar_type() == at::kBFloat16, "latent_attn_mfma: bf16 GPU tensors");
   TORCH_CHECK(q_lat.dim() == 3 && q_lat.stride(2) == 1 && out.dim() == 3 && out.stride(2) == 1 && q_rot.dim() == 3 &&
@@ -289,11 +290,20 @@ void latent_attn_mfma(at::Tensor q_lat, at::Tensor q_rot, at::Tensor cache, at::
                   items.scalar_type() == at::kInt && items.is_contiguous() && items.dim() == 2 && items.size(1) == 4 &&
                   positions.is_cuda() && positions.scalar_type() == at::kLong && positions.is_contiguous() &&
                   positions.numel() == T, "latent_attn_mfma: block tables / items / positions");
+  float *pop = nullptr, *pmlp = nullptr;
+  TORCH_CHECK(nsplit >= 1 && nsplit <= 64, "latent_attn_mfma: 1..64 key-range splits");
+  if (nsplit > 1) {
+    TORCH_CHECK(po.has_value() && pml.has_value() && po->is_cuda() && po->scalar_type() == at::kFloat &&
+                    po->is_contiguous() && po->numel() >= nsplit * H * T * R && pml->is_cuda() &&
+                    pml->scalar_type() == at::kFloat && pml->is_contiguous() && pml->numel() >= nsplit * H * T * 2,
+                "latent_attn_mfma: split workspaces fp32 [splits, H, T, R] and [splits, H, T, 2]");
+    pop = po->data_ptr<float>(); pmlp = pml->data_ptr<float>();
+  }
   HY_HIP(kafka_hy_latent_attn_mfma(q_lat.data_ptr(), q_lat.stride(0), q_lat.stride(1), q_rot.data_ptr(),
                                    q_rot.stride(0), q_rot.stride(1), cache.data_ptr(), cache_t.data_ptr(), (int)R,
                                    (int)rd, bt.data_ptr<int>(), (int)bt.stride(0), items.data_ptr<int>(),
                                    (int)items.size(0), positions.data_ptr<int64_t>(), (float)scale, out.data_ptr(),
-                                   out.stride(0), out.stride(1), (int)H, stream()));
+                                   out.stride(0), out.stride(1), (int)H, (int)nsplit, pop, pmlp, (int)T, stream()));
 }
 
 void conv_silu(at::Tensor proj, int64_t c0, at::Tensor w, at::Tensor b, at::Tensor tok_seg, at::Tensor seg,
@@ -393,7 +403,10 @@ void kafka_bind_hybrid(pybind11::module_& m) {
   m.def("hy_latent_prep", &latent_prep, py::arg("qgd"), py::arg("H"), py::arg("dim"), py::arg("rd"), py::arg("R"),
         py::arg("dkv_off"), py::arg("dkv_w"), py::arg("eps"), py::arg("positions"), py::arg("cos_sin"),
         py::arg("dims"), py::arg("cache"), py::arg("slots"), py::arg("q_rot"), py::arg("cache_t") = py::none());
-  m.def("hy_latent_attn_mfma", &latent_attn_mfma);
+  m.def("hy_latent_attn_mfma", &latent_attn_mfma, py::arg("q_lat"), py::arg("q_rot"), py::arg("cache"),
+        py::arg("cache_t"), py::arg("bt"), py::arg("items"), py::arg("tile_tokens"), py::arg("positions"),
+        py::arg("scale"), py::arg("out"), py::arg("nsplit") = 1, py::arg("po") = py::none(),
+        py::arg("pml") = py::none());
   m.def("hy_latent_mfma_ok", [](int page, int R, int rd) { return kafka_hy_latent_mfma_ok(page, R, rd) != 0; });
   m.def("hy_sigmoid_mul", &sigmoid_mul);
   m.def("hy_latent_attn", &latent_attn);

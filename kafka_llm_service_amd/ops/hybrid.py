@@ -101,17 +101,38 @@ def tile_tokens(heads: int) -> int:
     return max(1, MFMA_ROWS // heads)
 
 
+ATTN_SPLIT_WGS = 256   # workgroups a matrix-core attention launch should reach before its key ranges are left whole
+ATTN_SPLIT_MAX = 16
+
+
+def attn_splits(n_tiles: int, heads: int, max_keys: int) -> int:
+    """Key-range splits of a matrix-core attention launch: few tiles (a decode step's one tile per sequence) against
+    long contexts are dealt over more workgroups, each at least two 128-key blocks long; a merge pass combines them."""
+    wgs = n_tiles * -(-heads // MFMA_ROWS)
+    blocks = -(-max_keys // 128)
+    if wgs >= ATTN_SPLIT_WGS // 2 or blocks < 4:
+        return 1
+    return max(1, min(ATTN_SPLIT_MAX, ATTN_SPLIT_WGS // wgs, blocks // 2))
+
+
 def latent_attn(q_lat, q_rot, cache, block_tables, tok_seg, seg, positions, scale, out, cache_t=None,
-                tiles=None) -> None:
+                tiles=None, max_keys: int = 0) -> None:
     """Causal softmax attention of every row's heads over its sequence's cached [latent | rotated key] rows:
     out[h, t] = sum_j softmax_j((q_lat[h, t] . c_j + q_rot[t, h] . k_j) scale) c_j over the keys j <= position[t].
     With the transposed latent copy ``cache_t`` and ``tiles`` (int32 [n, 4] = (first row, tokens, segment, 0), at
     most ``tile_tokens(H)`` tokens of one segment each) bf16 runs on the matrix cores; else one wave per (row, 4
-    heads) on the vector units (fp32, odd sizes)."""
+    heads) on the vector units (fp32, odd sizes). ``max_keys`` (the step's longest context) lets a launch of few
+    tiles split its key ranges over more workgroups (``attn_splits``)."""
     if _gpu(q_lat):
         if cache_t is not None and tiles is not None and q_lat.dtype == torch.bfloat16:
-            ext().hy_latent_attn_mfma(q_lat, q_rot, cache, cache_t, block_tables, tiles, tile_tokens(q_lat.shape[0]),
-                                      positions, float(scale), out)
+            H, T, R = q_lat.shape
+            ns = attn_splits(tiles.shape[0], H, max_keys) if max_keys else 1
+            po = pml = None
+            if ns > 1:
+                po = torch.empty(ns, H, T, R, dtype=torch.float32, device=q_lat.device)
+                pml = torch.empty(ns, H, T, 2, dtype=torch.float32, device=q_lat.device)
+            ext().hy_latent_attn_mfma(q_lat, q_rot, cache, cache_t, block_tables, tiles, tile_tokens(H), positions,
+                                      float(scale), out, ns, po, pml)
         else:
             ext().hy_latent_attn(q_lat, q_rot, cache, block_tables, tok_seg, positions, float(scale), out)
     else:

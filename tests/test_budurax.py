@@ -308,6 +308,51 @@ def test_latent_attention_matrix_cores(R, rd, H):
         assert torch.allclose(ref[:, i].double().cpu(), want, atol=3e-3), (i, p)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("R,rd,H", [(64, 16, 3), (512, 64, 40)])
+def test_latent_attention_split_key_ranges(R, rd, H):
+    """A decode step of three sequences (1100, 300 and 5 cached keys): the launch deals each tile's key blocks over
+    several workgroups and merges them; sequences shorter than a split's range leave it empty."""
+    device = "cuda:0"
+    torch.manual_seed(7)
+    lens, page = [1100, 300, 5], 16
+    cache = torch.zeros(100, page, R + rd, dtype=torch.bfloat16, device=device)
+    perm = torch.randperm(100).tolist()
+    bt = torch.zeros(3, 80, dtype=torch.int32, device=device)
+    kvs, at = [], 0
+    for r, n in enumerate(lens):
+        kv = torch.nn.functional.normalize(torch.randn(n, R + rd), dim=-1).bfloat16()
+        kvs.append(kv)
+        need = -(-n // page)
+        pages = perm[at:at + need]
+        at += need
+        bt[r, :need] = torch.tensor(pages)
+        flat = cache.view(-1, R + rd)
+        for j in range(n):
+            flat[pages[j // page] * page + j % page] = kv[j].to(device)
+    cache_t = cache[:, :, :R].transpose(1, 2).contiguous()
+    seg, ts = _seg(device, [(1, n - 1, r) for r, n in enumerate(lens)])
+    positions = torch.tensor([n - 1 for n in lens], device=device)
+    tiles = torch.tensor([(r, 1, r, 0) for r in range(3)], dtype=torch.int32, device=device)
+    assert hops.attn_splits(3, H, max(lens)) > 1
+    q_lat, q_rot = torch.randn(H, 3, R).bfloat16(), torch.randn(3, H, rd).bfloat16()
+    out = torch.empty(H, 3, R, dtype=torch.bfloat16, device=device)
+    hops.latent_attn(q_lat.to(device), q_rot.to(device), cache, bt, ts, seg, positions, 0.5, out, cache_t, tiles,
+                     max_keys=max(lens))
+    for i, n in enumerate(lens):
+        kv = kvs[i].double()
+        sc = (q_lat[:, i].double() @ kv[:, :R].T + q_rot[i].double() @ kv[:, R:].T) * 0.5
+        want = torch.softmax(sc, -1) @ kv[:, :R]
+        assert torch.allclose(out[:, i].double().cpu(), want, atol=3e-3), i
+    # single dominant keys in the first, a middle and the last split
+    for j in (0, 640, 1099):
+        q = kvs[0][j].float() * 80.0
+        ql = q[:R][None, None].repeat(H, 3, 1).bfloat16().contiguous().to(device)
+        qr = q[R:][None, None].repeat(3, H, 1).bfloat16().contiguous().to(device)
+        hops.latent_attn(ql, qr, cache, bt, ts, seg, positions, 1.0, out, cache_t, tiles, max_keys=max(lens))
+        assert torch.allclose(out[:, 0].float().cpu(), kvs[0][j, :R].float().expand(H, R), atol=6e-3), j
+
+
 def cfg_m():
     """Sizes the matrix-core attention kernel takes (latent 64, rotary part 16), two attention layers sharing a cache."""
     ff = {"kind": "dense", "ff": 96}
