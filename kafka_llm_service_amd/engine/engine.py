@@ -466,7 +466,14 @@ class LLMEngine:
             if plan is not None:
                 batch, host, sampled = plan.batch, plan.host, plan.sampled
         T = host.T if host is not None else 0
-        got = agree((T, int(self.has_unfinished()), int(flag)) + tuple(extra))
+        try:
+            got = agree((T, int(self.has_unfinished()), int(flag)) + tuple(extra))
+        except Exception:
+            # the group did not answer (a peer is gone or late): if the step in flight already lost a peer in one of
+            # its collectives, that is the error to report (collect raises CollectiveError on its error word)
+            if self._inflight is not None:
+                self.runner.collect(self._inflight.launched)
+            raise
         t_max, busy, fl, ext = got[0], got[1], got[2], tuple(got[3:])
         cur, self._inflight = self._inflight, None
         if t_max > 0:

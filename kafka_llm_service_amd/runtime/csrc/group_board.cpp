@@ -16,6 +16,9 @@
 #include <fcntl.h>
 #include <pybind11/numpy.h>
 #include <pybind11/pybind11.h>
+
+#include <cstdio>
+#include <cstring>
 #include <sched.h>
 #include <signal.h>
 #include <sys/mman.h>
@@ -55,7 +58,22 @@ struct BoardHeader {
   BoardSlot slots[kBoardMaxRanks];
 };
 
-static bool board_pid_gone(int64_t pid) { return pid > 0 && kill((pid_t)pid, 0) != 0 && errno == ESRCH; }
+// a peer that no longer runs: no such process, or exited and not yet reaped by its parent (a zombie still answers
+// kill(pid, 0), and a parent that waits for the OTHER ranks would keep it one for as long as they wait for it)
+static bool board_pid_gone(int64_t pid) {
+  if (pid <= 0) return false;
+  if (kill((pid_t)pid, 0) != 0 && errno == ESRCH) return true;
+  char path[64];
+  snprintf(path, sizeof(path), "/proc/%lld/stat", (long long)pid);
+  FILE* f = fopen(path, "r");
+  if (f == nullptr) return false;
+  char buf[512];
+  const size_t n = fread(buf, 1, sizeof(buf) - 1, f);
+  fclose(f);
+  buf[n] = 0;
+  const char* p = strrchr(buf, ')');  // the state letter follows the parenthesised command name
+  return p != nullptr && p[1] == ' ' && (p[2] == 'Z' || p[2] == 'X');
+}
 
 class GroupBoard {
  public:
