@@ -660,32 +660,45 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(const AT* __restrict__ xb
   const int ypo = 2 * bufsz;            // yp [TB][TN][W] at sm[ypo]
   if (NP != N)
     for (int i = tid; i < 2 * TB * stride; i += nthr) sm[i] = 0.f;
-  // what this thread fetches of every block: (token in block, element) per slot, fixed for the whole scan
-  int ftok[SCAN_MAXL], fidx[SCAN_MAXL];
+  // what this thread fetches of every block, fixed for the whole scan: per slot the source address at block 0, its
+  // step per token (a row of xbc or of proj), the LDS offset it lands at, and the token it belongs to - so a fetch is
+  // one multiply-add and a load, a stash one store (the step-size slot also derives dA)
+  const AT* fsrc[SCAN_MAXL];
+  int fdst[SCAN_MAXL], ftok[SCAN_MAXL];  // ftok: token in block | 1 << 28 zero column | 1 << 29 step-size slot
 #pragma unroll
   for (int l = 0; l < SCAN_MAXL; ++l) {
     const int e = tid + l * nthr;
-    ftok[l] = e / per_tok;
-    fidx[l] = e - ftok[l] * per_tok;
-    if (ftok[l] >= TB) ftok[l] = 1 << 20;  // never fetched
+    const int tt = e / per_tok, idx = e - tt * per_tok;
+    const int64_t row = q0 + tt;
+    const AT* xr = xbc + row * xs;
+    int flags = 0;
+    if (idx < N) {
+      fsrc[l] = xr + inner + grp * N + idx;
+      fdst[l] = idx;
+    } else if (idx < 2 * N) {
+      fsrc[l] = xr + inner + (G + grp) * N + (idx - N);
+      fdst[l] = NP + (idx - N);
+    } else if (idx < 2 * N + W) {
+      const int pp = idx - 2 * N;
+      fsrc[l] = xr + h * P + pbase + min(pp, pw - 1);
+      fdst[l] = 2 * NP + pp;
+      if (pp >= pw) flags = 1 << 28;
+    } else {
+      fsrc[l] = proj + row * ps + dt_off + h;
+      fdst[l] = 2 * NP + W;
+      flags = 1 << 29;
+    }
+    fdst[l] += tt * stride;
+    ftok[l] = tt >= TB ? (1 << 27) : (tt | flags);  // beyond the block: never fetched
   }
   float pre[SCAN_MAXL];
   auto fetch = [&](int t0) {
     const int nt = min(TB, n - t0);
 #pragma unroll
     for (int l = 0; l < SCAN_MAXL; ++l) {
-      if (ftok[l] < nt) {
-        const int idx = fidx[l];
-        const int64_t row = q0 + t0 + ftok[l];
-        // one straight-line load per element (the address is selected, not the load)
-        const AT* xr = xbc + row * xs;
-        const AT* src = idx < N ? xr + inner + grp * N + idx
-                        : idx < 2 * N ? xr + inner + (G + grp) * N + (idx - N)
-                        : idx < 2 * N + W ? xr + h * P + pbase + min(idx - 2 * N, pw - 1)
-                                          : proj + row * ps + dt_off + h;
-        float v = ldf(src);
-        if (idx >= 2 * N && idx < 2 * N + W && idx - 2 * N >= pw) v = 0.f;
-        pre[l] = v;
+      if ((ftok[l] & 0xffffff) < nt && !(ftok[l] & (1 << 27))) {
+        const int64_t step = (ftok[l] & (1 << 29)) ? ps : xs;
+        pre[l] = ldf(fsrc[l] + (int64_t)t0 * step);
       }
     }
   };
@@ -693,16 +706,14 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(const AT* __restrict__ xb
     const int nt = min(TB, n - t0);
 #pragma unroll
     for (int l = 0; l < SCAN_MAXL; ++l) {
-      if (ftok[l] < nt) {
-        const int idx = fidx[l];
-        const int d = dsto + ftok[l] * stride;
-        if (idx == per_tok - 1) {
+      if ((ftok[l] & 0xffffff) < nt && !(ftok[l] & (1 << 27))) {
+        if (ftok[l] & (1 << 29)) {
           const float raw = pre[l] + bias;
           const float dt = raw > 20.f ? raw : log1pf(expf(raw));  // softplus
-          sm[d + 2 * NP + W] = dt;
-          sm[d + 2 * NP + W + 1] = expf(A * dt);
+          sm[dsto + fdst[l]] = dt;
+          sm[dsto + fdst[l] + 1] = expf(A * dt);
         } else {
-          sm[d + (idx < N ? idx : idx < 2 * N ? NP + (idx - N) : 2 * NP + (idx - 2 * N))] = pre[l];
+          sm[dsto + fdst[l]] = (ftok[l] & (1 << 28)) ? 0.f : pre[l];
         }
       }
     }
