@@ -290,8 +290,12 @@ class LLMEngine:
         for rid, toks, offs in entries:
             toks = [int(t) for t in toks]
             V = self.model_cfg.vocab_size
-            if not toks or min(toks) < 0 or max(toks) >= V:
-                raise ValueError(f"request {rid}: token ids must lie in [0, {V}) and a portion cannot be empty")
+            if not toks:  # nothing of this request in this step
+                if offs:
+                    raise ValueError(f"request {rid}: rows wanted of an empty portion")
+                continue
+            if min(toks) < 0 or max(toks) >= V:
+                raise ValueError(f"request {rid}: token ids must lie in [0, {V})")
             seq = self.requests.get(rid)
             if seq is None:
                 seq = Sequence(rid, toks, SamplingParams(max_tokens=1))

@@ -563,6 +563,24 @@ def test_other_sizes_and_no_extras(device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
+def test_models_of_one_layer_kind(device):
+    """Only Mamba-2 layers (the page pool stays unused), only attention layers (no recurrent matrices), one tap."""
+    ff = {"kind": "dense", "ff": 56}
+    only_m = {"architecture": "Budurax", "vocab": 131, "width": 40, "norm": {"eps": 1e-6},
+              "layers": [{"type": "mamba2", "mixer": _mamba(2, 10, 6, 2, 1, 1), "mlp": ff},
+                         {"type": "mamba2", "mixer": _mamba(4, 5, 3, 1, 2, 8), "mlp": None}]}
+    only_a = {"architecture": "Budurax", "vocab": 131, "width": 40, "norm": {"eps": 1e-6}, "token_side": {"dim": 3},
+              "layers": [{"type": "latent_attention", "mixer": _attn(2, 8, 4, 4, 6, 12), "mlp": None},
+                         {"type": "latent_attention", "mixer": _attn(7, 4, 4, 4, 3, 12, kv_from=0), "mlp": ff}]}
+    for cfg in (only_m, only_a):
+        b = Bench(cfg, seed=21)
+        t = toks(50, 131, 8)
+        eng = b.engine(device)
+        assert rel_err(feed_all(eng, "w", t, [50]), b.oracle(t)) < TOL["float32"]
+        assert rel_err(feed_all(eng, "c", t, [7, 2, 20, 1]), b.oracle(t)) < TOL["float32"]
+
+
+@pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("cuts", [[1], [2], [3, 2], [16], [17, 15, 1, 2], [31, 1, 1, 1, 33], [64, 2]])
 def test_portions_and_decoding(bench_sharp, device, cuts):
     """Prompt portions of several sizes (down to two tokens, [1] = everything decoded token by token: 100 steps) give
