@@ -127,6 +127,171 @@ __global__ __launch_bounds__(NT) void add_ln_kernel(float* __restrict__ x, int64
   }
 }
 
+// ---- the same three row kernels with the row held in registers (d <= NV * 256) -------------------------------------
+// A step of few rows (a decode step) has few workgroups, so these kernels are latency-bound: every pass over a row
+// that goes back to memory is a dependent round trip. Here each row is loaded once (all its loads in flight together,
+// the previous row's and the second operand's too) and the statistics, the second norm and the outputs come from
+// registers. The sums run over the same elements in the same order as in the generic kernels above.
+template <int NV>
+__device__ __forceinline__ void reg_stats(const float (&v)[NV], int d, float eps, float* red, float& mean, float& rstd) {
+  float s = 0.f;
+#pragma unroll
+  for (int k = 0; k < NV; ++k)
+    if ((int)threadIdx.x + k * NT < d) s += v[k];
+  mean = block_sum<NT>(s, red) / (float)d;
+  float q = 0.f;
+#pragma unroll
+  for (int k = 0; k < NV; ++k)
+    if ((int)threadIdx.x + k * NT < d) {
+      const float c = v[k] - mean;
+      q += c * c;
+    }
+  rstd = inv_sqrt(block_sum<NT>(q, red) / (float)d + eps);
+}
+
+template <typename AT, int NV>
+__global__ __launch_bounds__(NT) void ln_shift_reg_kernel(const float* __restrict__ x, int64_t xs,
+                                                          const AT* __restrict__ w, const AT* __restrict__ b, float eps,
+                                                          AT* __restrict__ out, int64_t os, int d,
+                                                          const AT* __restrict__ mu, const int* __restrict__ tok_seg,
+                                                          const int* __restrict__ seg, const float* __restrict__ state,
+                                                          float* __restrict__ last) {
+  __shared__ float red[NT / 64];
+  const int64_t t = blockIdx.x;
+  const float* xr = x + t * xs;
+  bool first = true, is_last = false;
+  int sg = 0, p0 = 0, slot = 0;
+  if (mu != nullptr) {
+    sg = tok_seg[t];
+    const int q0 = seg[4 * sg], n = seg[4 * sg + 1];
+    p0 = seg[4 * sg + 2];
+    slot = seg[4 * sg + 3];
+    first = (t == q0);
+    is_last = (t == q0 + n - 1);
+  }
+  float v[NV], pv[NV], wv[NV], bv[NV];
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int i = threadIdx.x + k * NT;
+    const bool in = i < d;
+    v[k] = in ? xr[i] : 0.f;
+    wv[k] = in ? ldf(w + i) : 0.f;
+    bv[k] = in ? ldf(b + i) : 0.f;
+    pv[k] = 0.f;
+    if (mu != nullptr && in) pv[k] = first ? (p0 > 0 ? state[(int64_t)slot * d + i] : 0.f) : xr[i - xs];
+  }
+  float mean, rstd, mean2 = 0.f, rstd2 = 0.f;
+  reg_stats<NV>(v, d, eps, red, mean, rstd);
+  if (mu != nullptr && !first) reg_stats<NV>(pv, d, eps, red, mean2, rstd2);  // (uniform per workgroup)
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int i = threadIdx.x + k * NT;
+    if (i < d) {
+      const float h = (v[k] - mean) * rstd * wv[k] + bv[k];
+      if (mu == nullptr) {
+        stf(out + t * os + i, h);
+      } else {
+        const float prev = first ? pv[k] : (pv[k] - mean2) * rstd2 * wv[k] + bv[k];
+        stf(out + t * os + i, h + (prev - h) * ldf(mu + i));
+        if (is_last) last[(int64_t)sg * d + i] = h;
+      }
+    }
+  }
+}
+
+template <typename AT, int NV, int MODE>
+__global__ __launch_bounds__(NT) void add_ln_reg_kernel(float* __restrict__ x, int64_t xs, const AT* __restrict__ y,
+                                                        int64_t ys, const AT* __restrict__ w,
+                                                        const AT* __restrict__ b, float eps, int d,
+                                                        AT* __restrict__ out2, int64_t os, const AT* __restrict__ w2,
+                                                        const AT* __restrict__ b2) {
+  __shared__ float red[NT / 64];
+  const int64_t t = blockIdx.x;
+  float yv[NV], xv[NV];
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int i = threadIdx.x + k * NT;
+    yv[k] = i < d ? ldf(y + t * ys + i) : 0.f;
+    xv[k] = i < d ? x[t * xs + i] : 0.f;
+  }
+  float mean, rstd;
+  reg_stats<NV>(yv, d, eps, red, mean, rstd);
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int i = threadIdx.x + k * NT;
+    if (i < d) {
+      xv[k] = xv[k] + ((yv[k] - mean) * rstd * ldf(w + i) + ldf(b + i));
+      x[t * xs + i] = xv[k];
+      if constexpr (MODE == 2) stf(out2 + t * os + i, xv[k]);
+    }
+  }
+  if constexpr (MODE == 1) {
+    float m2, r2;
+    reg_stats<NV>(xv, d, eps, red, m2, r2);
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int i = threadIdx.x + k * NT;
+      if (i < d) stf(out2 + t * os + i, (xv[k] - m2) * r2 * ldf(w2 + i) + ldf(b2 + i));
+    }
+  }
+}
+
+template <typename AT, int NV>
+__global__ __launch_bounds__(NT) void side_dwa_reg_kernel(float* __restrict__ x, const AT* __restrict__ y, int64_t ys,
+                                                          const AT* __restrict__ sw, float eps,
+                                                          float* __restrict__ stack, int layer,
+                                                          const float* __restrict__ dwa, int64_t T, int d) {
+  __shared__ float red[NT / 64];
+  const int64_t t = blockIdx.x;
+  const int64_t plane = T * d;
+  float xv[NV], yv[NV];
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int i = threadIdx.x + k * NT;
+    xv[k] = i < d ? x[t * d + i] : 0.f;
+    yv[k] = (y != nullptr && i < d) ? ldf(y + t * ys + i) : 0.f;
+  }
+  if (y != nullptr) {
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) s += yv[k] * yv[k];  // (zeros beyond d)
+    const float r = inv_sqrt(block_sum<NT>(s, red) / (float)d + eps);
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int i = threadIdx.x + k * NT;
+      if (i < d) xv[k] += yv[k] * r * ldf(sw + i);
+    }
+  }
+  if (stack != nullptr) {
+    float a[NV];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int i = threadIdx.x + k * NT;
+      if (i < d) stack[(int64_t)(layer + 1) * plane + t * d + i] = xv[k];
+      a[k] = 0.f;
+    }
+    if (dwa != nullptr) {
+      for (int j = 0; j <= layer; ++j) {  // one plane per turn, the row's NV loads of it in flight together
+        const float c = dwa[j];
+        const float* pj = stack + (int64_t)j * plane + t * d;
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+          const int i = threadIdx.x + k * NT;
+          if (i < d) a[k] += c * pj[i];
+        }
+      }
+      const float c = dwa[layer + 1];
+#pragma unroll
+      for (int k = 0; k < NV; ++k) xv[k] = a[k] + c * xv[k];
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int i = threadIdx.x + k * NT;
+    if (i < d) x[t * d + i] = xv[k];
+  }
+}
+
 template <typename AT>
 __global__ void gelu_mul_kernel(const AT* __restrict__ gu, int64_t gs, AT* __restrict__ out, int64_t T, int F) {
   const int64_t n = T * F;
@@ -922,8 +1087,15 @@ hipError_t kafka_hy_ln_shift(int f32, const float* x, int64_t xs, const void* w,
                              int64_t os, int T, int d, const void* mu, const int* tok_seg, const int* seg,
                              const float* state, float* last, hipStream_t st) {
   if (T <= 0) return hipSuccess;
-  DISPATCH_AT(f32, ln_shift_kernel<AT><<<T, NT, 0, st>>>(x, xs, (const AT*)w, (const AT*)b, eps, (AT*)out, os, d,
-                                                        (const AT*)mu, tok_seg, seg, state, last));
+  DISPATCH_AT(f32, {
+    auto a = [&](auto k) {
+      k<<<T, NT, 0, st>>>(x, xs, (const AT*)w, (const AT*)b, eps, (AT*)out, os, d, (const AT*)mu, tok_seg, seg, state,
+                          last);
+    };
+    if (d <= 4 * NT) a(ln_shift_reg_kernel<AT, 4>);
+    else if (d <= 16 * NT) a(ln_shift_reg_kernel<AT, 16>);
+    else a(ln_shift_kernel<AT>);
+  });
   return hipGetLastError();
 }
 
@@ -943,7 +1115,15 @@ hipError_t kafka_hy_add_ln(int f32, float* x, int64_t xs, const void* y, int64_t
       k<<<T, NT, 0, st>>>(x, xs, (const AT*)y, ys, (const AT*)w, (const AT*)b, eps, d, (AT*)out2, os, (const AT*)w2,
                           (const AT*)b2);
     };
-    if (mode == 0) a(add_ln_kernel<AT, 0>);
+    if (d <= 4 * NT) {
+      if (mode == 0) a(add_ln_reg_kernel<AT, 4, 0>);
+      else if (mode == 1) a(add_ln_reg_kernel<AT, 4, 1>);
+      else a(add_ln_reg_kernel<AT, 4, 2>);
+    } else if (d <= 16 * NT) {
+      if (mode == 0) a(add_ln_reg_kernel<AT, 16, 0>);
+      else if (mode == 1) a(add_ln_reg_kernel<AT, 16, 1>);
+      else a(add_ln_reg_kernel<AT, 16, 2>);
+    } else if (mode == 0) a(add_ln_kernel<AT, 0>);
     else if (mode == 1) a(add_ln_kernel<AT, 1>);
     else a(add_ln_kernel<AT, 2>);
   });
@@ -967,8 +1147,12 @@ hipError_t kafka_hy_side_gate(int f32, const void* sg, int64_t ss, const int64_t
 hipError_t kafka_hy_side_dwa(int f32, float* x, const void* y, int64_t ys, const void* sw, float eps, float* stack,
                              int layer, const float* dwa, int64_t T, int d, hipStream_t st) {
   if (T <= 0) return hipSuccess;
-  DISPATCH_AT(f32, side_dwa_kernel<AT><<<(int)T, NT, 0, st>>>(x, (const AT*)y, ys, (const AT*)sw, eps, stack, layer,
-                                                              dwa, T, d));
+  DISPATCH_AT(f32, {
+    auto a = [&](auto k) { k<<<(int)T, NT, 0, st>>>(x, (const AT*)y, ys, (const AT*)sw, eps, stack, layer, dwa, T, d); };
+    if (d <= 4 * NT) a(side_dwa_reg_kernel<AT, 4>);
+    else if (d <= 16 * NT) a(side_dwa_reg_kernel<AT, 16>);
+    else a(side_dwa_kernel<AT>);
+  });
   return hipGetLastError();
 }
 

@@ -138,9 +138,10 @@ def test_rotary_table(device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-def test_norm_and_shift(device):
+@pytest.mark.parametrize("d", [70, 2500, 4200])   # (the kernels keep rows of up to 1024 / 4096 values in registers)
+def test_norm_and_shift(device, d):
     torch.manual_seed(0)
-    d, T = 70, 9
+    T = 9
     x = torch.randn(T, d) * 3 + 1
     w, b, mu = torch.randn(d), torch.randn(d), torch.rand(d)
     want = plain.token_shift(plain.layer_norm(x.double(), w.double(), b.double(), 1e-5), mu.double())
@@ -168,9 +169,10 @@ def test_norm_and_shift(device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-def test_add_norm_gelu_side_depth(device):
+@pytest.mark.parametrize("d", [52, 2500, 4200])
+def test_add_norm_gelu_side_depth(device, d):
     torch.manual_seed(1)
-    T, d, F, sd, V = 6, 52, 30, 5, 40
+    T, F, sd, V = 6, 30, 5, 40
     x, y = torch.randn(T, d), torch.randn(T, d) * 2
     w, b, w2, b2 = (torch.randn(d) for _ in range(4))
     xd = x.clone().to(device)
