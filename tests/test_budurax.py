@@ -685,3 +685,34 @@ def test_config_registry_and_checkpoint(tmp_path):
         bx.BuduraxLM(b.mc, "cpu").load_tensors(bad)
     assert get_config("budurax-tiny").arch == "budurax"
     assert math.isclose(get_config("budurax-tiny").norm_eps, 1e-6)
+
+
+def test_trace_runner_command_line(tmp_path):
+    """bin/trace_run as a program (reference ops on the CPU): a checkpoint folder, three steps on standard input - a
+    new request, two requests in one step, a step in which nothing is wanted - then the logits files, the "done"
+    lines and the exit code."""
+    import json
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    import numpy as np
+
+    root = Path(__file__).resolve().parents[1]
+    b = Bench(cfg_b(), seed=14)
+    bx.save_checkpoint(b.mc, b.W, tmp_path / "m")
+    t, u = toks(21, 97, 1), toks(6, 97, 2)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": t[:9], "want": [0, 8]}], "end": []},
+             {"step": 1, "entries": [{"id": "b", "tokens": u, "want": [5]}, {"id": "a", "tokens": t[9:20], "want": []}],
+              "end": ["b"]},
+             {"step": 2, "entries": [{"id": "a", "tokens": t[20:], "want": [0]}], "end": ["a"]}]
+    out = subprocess.run([sys.executable, str(root / "bin/trace_run"), "--model", str(tmp_path / "m"), "--dtype",
+                          "float32", "--out", str(tmp_path / "o"), "--max-tokens", "64", "--device", "cpu"],
+                         input="".join(json.dumps(x) + "\n" for x in steps), capture_output=True, text=True,
+                         timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    assert [ln for ln in out.stdout.splitlines() if ln.startswith("done")] == ["done 0", "done 1", "done 2"]
+    got = {n: torch.from_numpy(np.fromfile(tmp_path / "o" / f"{n}.f32", dtype="<f4").reshape(-1, 97)) for n in range(3)}
+    assert rel_err(got[0], b.oracle(t)[[0, 8]]) < TOL["float32"]
+    assert rel_err(got[1], b.oracle(u)[[5]]) < TOL["float32"]
+    assert rel_err(got[2], b.oracle(t)[[20]]) < TOL["float32"]
