@@ -305,6 +305,9 @@ class LLMEngine:
                     raise RuntimeError(f"request {rid} has uncomputed tokens")
                 seq.prompt_ids.extend(toks)
                 self.kvm.append_tokens(seq.seq_id, toks)
+            if seq.total_len > self.cfg.max_model_len:
+                # positions index tables sized for max_model_len (rotary cos / sin): refuse instead of reading past them
+                raise ValueError(f"request {rid}: {seq.total_len} tokens exceed max_model_len={self.cfg.max_model_len}")
             portions.append((seq, len(toks)))
             want[seq.seq_id] = [int(o) for o in offs]
         logits = None
