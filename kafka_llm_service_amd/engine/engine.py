@@ -297,6 +297,10 @@ class LLMEngine:
             if min(toks) < 0 or max(toks) >= V:
                 raise ValueError(f"request {rid}: token ids must lie in [0, {V})")
             seq = self.requests.get(rid)
+            n_new = (seq.total_len if seq is not None else 0) + len(toks)
+            if n_new > self.cfg.max_model_len:
+                # positions index tables sized for max_model_len (rotary cos / sin): refuse instead of reading past them
+                raise ValueError(f"request {rid}: {n_new} tokens exceed max_model_len={self.cfg.max_model_len}")
             if seq is None:
                 seq = Sequence(rid, toks, SamplingParams(max_tokens=1))
                 self.requests[rid] = seq
@@ -305,9 +309,6 @@ class LLMEngine:
                     raise RuntimeError(f"request {rid} has uncomputed tokens")
                 seq.prompt_ids.extend(toks)
                 self.kvm.append_tokens(seq.seq_id, toks)
-            if seq.total_len > self.cfg.max_model_len:
-                # positions index tables sized for max_model_len (rotary cos / sin): refuse instead of reading past them
-                raise ValueError(f"request {rid}: {seq.total_len} tokens exceed max_model_len={self.cfg.max_model_len}")
             portions.append((seq, len(toks)))
             want[seq.seq_id] = [int(o) for o in offs]
         logits = None
