@@ -593,6 +593,29 @@ def moe_route(logits: torch.Tensor, k: int) -> MoERouting:
     return MoERouting(tw, te, pt, pw, eo, to, E)
 
 
+def moe_sort(topk_w: torch.Tensor, topk_e: torch.Tensor, num_experts: int) -> MoERouting:
+    """MoERouting of entries routed elsewhere (weights fp32 [T, k], expert ids int32 [T, k]): the stable sort by expert
+    of ``moe_route`` alone, for any number of experts and choices."""
+    T, k = topk_e.shape
+    dev = topk_e.device
+    if _gpu(topk_e):
+        pt = torch.empty(T * k, dtype=torch.int32, device=dev)
+        pw = torch.empty(T * k, dtype=torch.float32, device=dev)
+        eo = torch.empty(num_experts + 1, dtype=torch.int32, device=dev)
+        to = torch.empty(num_experts + 1, dtype=torch.int32, device=dev)
+        ext().moe_sort(topk_w, topk_e, int(num_experts), GG_BM, pt, pw, eo, to)
+        return MoERouting(topk_w, topk_e, pt, pw, eo, to, num_experts)
+    flat = topk_e.reshape(-1).long()
+    perm = torch.argsort(flat, stable=True)
+    counts = torch.bincount(flat, minlength=num_experts)
+    eo = torch.zeros(num_experts + 1, dtype=torch.int32)
+    eo[1:] = torch.cumsum(counts, 0)
+    to = torch.zeros(num_experts + 1, dtype=torch.int32)
+    to[1:] = torch.cumsum((counts + GG_BM - 1) // GG_BM, 0)
+    return MoERouting(topk_w, topk_e, (perm // k).to(torch.int32), topk_w.reshape(-1)[perm].float(), eo, to,
+                      num_experts)
+
+
 def grouped_gemm(x: torch.Tensor, w: torch.Tensor, r: MoERouting, gather: bool, e_lo: int = 0,
                  y: torch.Tensor | None = None, combine_out: torch.Tensor | None = None) -> torch.Tensor:
     """Per expert segment of the routed entries: Y = X_e . W_e^T (W = [E_local, N, K], experts [e_lo, e_lo+E_local)).

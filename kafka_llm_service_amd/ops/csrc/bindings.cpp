@@ -768,6 +768,23 @@ static void moe_route(at::Tensor logits, int64_t k, int64_t bm, at::Tensor topk_
                                    expert_off.data_ptr<int>(), tile_off.data_ptr<int>(), cur_stream()));
 }
 
+// the sort of moe_route alone, for entries routed elsewhere (topk_w / topk_e [T, k] are inputs; expert ids in [0, E))
+static void moe_sort(at::Tensor topk_w, at::Tensor topk_e, int64_t E, int64_t bm, at::Tensor perm_tok,
+                     at::Tensor perm_w, at::Tensor expert_off, at::Tensor tile_off) {
+  CHECK_CUDA(topk_w); CHECK_DT(topk_w, at::kFloat); CHECK_DT(perm_w, at::kFloat);
+  CHECK_DT(topk_e, at::kInt); CHECK_DT(perm_tok, at::kInt); CHECK_DT(expert_off, at::kInt); CHECK_DT(tile_off, at::kInt);
+  TORCH_CHECK(topk_w.dim() == 2 && topk_e.sizes() == topk_w.sizes() && topk_w.is_contiguous() && topk_e.is_contiguous(),
+              "moe_sort: topk [T, k]");
+  const int64_t T = topk_w.size(0), k = topk_w.size(1);
+  TORCH_CHECK(T >= 1 && k >= 1 && k <= E && E <= 4096, "moe_sort: unsupported T/E/k");
+  TORCH_CHECK(perm_tok.numel() == T * k && perm_w.numel() == T * k && expert_off.numel() == E + 1 &&
+                  tile_off.numel() == E + 1 && perm_tok.is_contiguous() && perm_w.is_contiguous(),
+              "moe_sort: output sizes");
+  CHECK_HIP(kafka_launch_moe_route(nullptr, 0, (int)T, (int)E, (int)k, (int)bm, topk_w.data_ptr<float>(),
+                                   topk_e.data_ptr<int>(), perm_tok.data_ptr<int>(), perm_w.data_ptr<float>(),
+                                   expert_off.data_ptr<int>(), tile_off.data_ptr<int>(), cur_stream()));
+}
+
 // Y (or out += w * Y) = X_e . W_e^T per expert segment of the routed entries; W = [e_n, N, K] local experts
 static void grouped_gemm(at::Tensor x, at::Tensor w, at::Tensor perm_tok, at::Tensor perm_w, at::Tensor expert_off,
                          at::Tensor tile_off, int64_t e_lo, int64_t max_tiles, bool gather,
@@ -1025,6 +1042,7 @@ PYBIND11_MODULE(_kafka_ops, m) {
   m.def("wstream_grouped", &wstream_grouped, py::arg("x"), py::arg("wt"), py::arg("perm_tok"), py::arg("perm_w"),
         py::arg("expert_off"), py::arg("e_lo"), py::arg("max_rows"), py::arg("gather"), py::arg("y"), py::arg("out"),
         py::arg("pin") = true);
+  m.def("moe_sort", &moe_sort);
   m.def("moe_route", &moe_route);
   m.def("cu_mask_stream", &cu_mask_stream);
   m.def("stream_cu_mask", &stream_cu_mask);

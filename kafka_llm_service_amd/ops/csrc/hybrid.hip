@@ -19,7 +19,7 @@
 //   latent_attn     all heads of a row against the row's cached [latent | rotary key] rows: one wave per (row, 4
 //                   heads), the 64 lanes across the row's dimensions, online softmax, the value pass reusing the key
 //                   registers (the values ARE the latent part of the key row)
-//   conv_silu       causal short convolution + silu with a per-slot tail of raw inputs
+//   short_conv      causal short convolution (optional bias, silu, residual) with a per-slot tail of raw inputs
 //   ssm_scan        the state-space recurrence, one workgroup per (segment, head, column slice), an 8 x 4 state block
 //                   per thread in registers, B / C / x / dt of the next tokens staged through LDS, double buffered
 //   gated_norm      y * silu(z), RMS norm in groups, weight
@@ -731,18 +731,20 @@ __global__ void latent_merge_kernel(const float* __restrict__ po, const float* _
 }
 
 // ---- Mamba-2 ---------------------------------------------------------------------------------------------------------
+// out = act(b + sum_k w[:, k] u_(t - taps + 1 + k)) (+ u_t): b may be null, act = silu or none
 template <typename AT>
-__global__ void conv_silu_kernel(const AT* __restrict__ proj, int64_t ps, int c0, const AT* __restrict__ w,
-                                 const AT* __restrict__ b, int C, int taps, const int* __restrict__ tok_seg,
-                                 const int* __restrict__ seg, const AT* __restrict__ state, AT* __restrict__ out,
-                                 int64_t T) {
+__global__ void short_conv_kernel(const AT* __restrict__ proj, int64_t ps, int c0, const AT* __restrict__ w,
+                                  const AT* __restrict__ b, int C, int taps, const int* __restrict__ tok_seg,
+                                  const int* __restrict__ seg, const AT* __restrict__ state, AT* __restrict__ out,
+                                  int64_t T, int silu, int residual) {
   const int64_t n = T * C;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
     const int64_t t = i / C;
     const int c = (int)(i - t * C);
     const int sg = tok_seg[t];
     const int q0 = seg[4 * sg], p0 = seg[4 * sg + 2], slot = seg[4 * sg + 3];
-    float a = ldf(b + c);
+    float a = b ? ldf(b + c) : 0.f;
+    float own = 0.f;
     for (int k = 0; k < taps; ++k) {
       const int64_t src = t - (taps - 1 - k);
       float u = 0.f;
@@ -753,8 +755,11 @@ __global__ void conv_silu_kernel(const AT* __restrict__ proj, int64_t ps, int c0
         if (si >= 0) u = ldf(state + ((int64_t)slot * (taps - 1) + si) * C + c);
       }
       a += u * ldf(w + (int64_t)c * taps + k);
+      own = u;
     }
-    stf(out + i, a / (1.0f + expf(-a)));
+    if (silu) a = a / (1.0f + expf(-a));
+    if (residual) a += own;
+    stf(out + i, a);
   }
 }
 
@@ -768,7 +773,7 @@ __global__ void conv_state_kernel(const AT* __restrict__ proj, int64_t ps, int c
   const int r = (int)(i / C), c = (int)(i - (int64_t)r * C);
   const int q0 = seg[4 * r], n = seg[4 * r + 1], p0 = seg[4 * r + 2], slot = seg[4 * r + 3];
   AT* st = state + (int64_t)slot * (taps - 1) * C + c;
-  AT v[8];
+  AT v[16];
   for (int k = 0; k < taps - 1; ++k) {
     const int at = n + k;  // index in (old tail ++ inputs)
     if (at < taps - 1)
@@ -1238,13 +1243,13 @@ hipError_t kafka_hy_latent_attn_mfma(const void* q_lat, int64_t ql_h, int64_t ql
   return hipGetLastError();
 }
 
-hipError_t kafka_hy_conv_silu(int f32, const void* proj, int64_t ps, int c0, const void* w, const void* b, int C,
-                              int taps, const int* tok_seg, const int* seg, int R, void* state, void* out, int64_t T,
-                              hipStream_t st) {
-  if (T <= 0 || taps > 8) return taps > 8 ? hipErrorInvalidValue : hipSuccess;
+hipError_t kafka_hy_short_conv(int f32, const void* proj, int64_t ps, int c0, const void* w, const void* b, int C,
+                               int taps, const int* tok_seg, const int* seg, int R, void* state, void* out, int64_t T,
+                               int silu, int residual, hipStream_t st) {
+  if (T <= 0 || C <= 0 || taps > 16 || taps < 1) return (taps > 16 || taps < 1) ? hipErrorInvalidValue : hipSuccess;
   DISPATCH_AT(f32, {
-    conv_silu_kernel<AT><<<ew_grid(T * C), 256, 0, st>>>((const AT*)proj, ps, c0, (const AT*)w, (const AT*)b, C, taps,
-                                                         tok_seg, seg, (const AT*)state, (AT*)out, T);
+    short_conv_kernel<AT><<<ew_grid(T * C), 256, 0, st>>>((const AT*)proj, ps, c0, (const AT*)w, (const AT*)b, C, taps,
+                                                          tok_seg, seg, (const AT*)state, (AT*)out, T, silu, residual);
     if (taps > 1)
       conv_state_kernel<AT><<<(int)(((int64_t)R * C + 255) / 256), 256, 0, st>>>((const AT*)proj, ps, c0, C, taps, seg,
                                                                                 (AT*)state, R);

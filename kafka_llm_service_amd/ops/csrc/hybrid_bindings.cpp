@@ -34,9 +34,9 @@ hipError_t kafka_hy_latent_attn(int f32, const void* q_lat, int64_t ql_h, int64_
                                 int64_t qr_h, const void* cache, int page, int R, int rd, const int* bt, int bt_stride,
                                 const int* tok_seg, const int64_t* positions, float scale, void* out, int64_t o_h,
                                 int64_t o_t, int T, int H, hipStream_t st);
-hipError_t kafka_hy_conv_silu(int f32, const void* proj, int64_t ps, int c0, const void* w, const void* b, int C,
-                              int taps, const int* tok_seg, const int* seg, int R, void* state, void* out, int64_t T,
-                              hipStream_t st);
+hipError_t kafka_hy_short_conv(int f32, const void* proj, int64_t ps, int c0, const void* w, const void* b, int C,
+                               int taps, const int* tok_seg, const int* seg, int R, void* state, void* out, int64_t T,
+                               int silu, int residual, hipStream_t st);
 int kafka_hy_scan_groups(int P, int N);
 hipError_t kafka_hy_ssm_scan(int f32, const void* xbc, int64_t xs, const void* proj, int64_t ps, int dt_off,
                              const float* dt_bias, const float* A_log, const float* Dp, int heads, int P, int N, int G,
@@ -46,6 +46,50 @@ hipError_t kafka_hy_ssm_combine(int f32, const void* proj, int64_t ps, int dt_of
                                 float* tmp, float* state, hipStream_t st);
 hipError_t kafka_hy_gated_norm(int f32, const float* y, int64_t ys, const void* z, int64_t zs, const void* w, int inner,
                                int groups, float eps, void* out, int64_t os, int64_t T, hipStream_t st);
+
+// gated mixers (hybrid_gated.hip)
+hipError_t kafka_hy_rms_norm(int f32, const float* x, int64_t xs, const void* w, float eps, void* out, int64_t os,
+                             int T, int d, hipStream_t st);
+hipError_t kafka_hy_kv_store(int f32, const void* src, int64_t ss, int k_off, int v_off, int Ck, int Cv, void* kc,
+                             void* vt, const int64_t* slots, int64_t T, hipStream_t st);
+int kafka_hy_sigmoid_attn_max_d();
+int kafka_hy_sigmoid_attn_max_dv();
+hipError_t kafka_hy_sigmoid_attn(int f32, const void* q, int64_t qs, int q_off, const void* kc, const void* vt,
+                                 const int* bt, int bt_stride, const int* tok_seg, const int64_t* positions, int H,
+                                 int G, int D, int Dv, float scale, float softcap, float t_coef, double t_every,
+                                 const float* r1, const float* r2, const float* pb, void* out, int64_t os, int64_t T,
+                                 hipStream_t st);
+int kafka_hy_sigmoid_attn_mfma_ok(int page, int D, int Dv, int rep);
+hipError_t kafka_hy_sigmoid_attn_mfma(const void* q, int64_t qs, int q_off, const void* kc, const void* vt,
+                                      const int* bt, int bt_stride, const int* items, int n_items,
+                                      const int64_t* positions, int H, int G, int D, int Dv, float scale,
+                                      float softcap, float t_coef, double t_every, const float* r1, const float* r2,
+                                      const float* pb, void* out, int64_t os, int nsplit, float* po, int64_t T,
+                                      hipStream_t st);
+hipError_t kafka_hy_rglru_scan(int f32, const float* gates, int64_t gs, const void* proj, int64_t ps, const void* u,
+                               int64_t us, const float* rate, const int* seg, int R, float* state, void* out,
+                               int64_t os, int W, hipStream_t st);
+int kafka_hy_rglru_chunk();
+hipError_t kafka_hy_rglru_scan_chunked(int f32, float* gates, int64_t gs, const void* proj, int64_t ps, const void* u,
+                                       int64_t us, const float* rate, const int* seg, int R, int nch, float* ab,
+                                       float* state, void* out, int64_t os, int64_t T, int W, hipStream_t st);
+int kafka_hy_mlstm_max_d();
+hipError_t kafka_hy_mlstm_scan(int f32, const void* qkv, int64_t qs, const float* gates, int64_t gs, int H, int D,
+                               int Dv, float cap, const int* seg, int R, float* S, float* nrm, float* mx, float* out,
+                               int64_t os, hipStream_t st);
+hipError_t kafka_hy_head_norm_gate(int f32, const float* o, int64_t os_, const void* w, const void* g, int64_t gs,
+                                   int g_off, int H, int Dv, float eps, void* out, int64_t outs, int64_t T,
+                                   hipStream_t st);
+int kafka_hy_router_max_e();
+int kafka_hy_router_max_k();
+hipError_t kafka_hy_moe_topk(const float* logits, int64_t ls, int E, int k, float* tw, int* te, int64_t T,
+                             hipStream_t st);
+int kafka_hy_moe_rows_max_d();
+hipError_t kafka_hy_moe_rows(int f32, const void* h, int64_t hs, const void* wgu, const void* wd, const float* tw,
+                             const int* te, int d, int F, int k, void* a, float* out, int64_t os, int64_t T,
+                             hipStream_t st);
+hipError_t kafka_hy_add2(int f32, float* x, int64_t xs, const void* y1, int64_t s1, const void* y2, int64_t s2,
+                         int y2_f32, int64_t T, int d, const void* w, float eps, void* out, int64_t os, hipStream_t st);
 }
 
 namespace {
@@ -306,23 +350,25 @@ void latent_attn_mfma(at::Tensor q_lat, at::Tensor q_rot, at::Tensor cache, at::
                                    out.stride(0), out.stride(1), (int)H, (int)nsplit, pop, pmlp, (int)T, stream()));
 }
 
-void conv_silu(at::Tensor proj, int64_t c0, at::Tensor w, at::Tensor b, at::Tensor tok_seg, at::Tensor seg,
-               at::Tensor state, at::Tensor out) {
+void short_conv(at::Tensor proj, int64_t c0, at::Tensor w, OptT b, at::Tensor tok_seg, at::Tensor seg,
+                at::Tensor state, at::Tensor out, bool silu, bool residual) {
   rows2d(proj, "proj");
   const int f32 = act_f32(proj);
-  same_act(f32, {&w, &b, &state, &out});
+  same_act(f32, {&w, &state, &out});
   const int64_t T = proj.size(0);
-  TORCH_CHECK(w.is_contiguous() && w.dim() == 2, "conv_silu: w [C, taps]");
+  TORCH_CHECK(w.is_contiguous() && w.dim() == 2, "short_conv: w [C, taps]");
   const int64_t C = w.size(0), taps = w.size(1);
-  vec(b, C, "conv bias");
+  if (b.has_value()) { same_act(f32, {&*b}); vec(*b, C, "conv bias"); }
   segs(tok_seg, seg, T);
-  TORCH_CHECK(taps >= 1 && taps <= 8 && c0 >= 0 && c0 + C <= proj.size(1) && out.is_contiguous() && out.dim() == 2 &&
-                  out.size(0) == T && out.size(1) == C, "conv_silu: shapes");
+  TORCH_CHECK(taps >= 1 && taps <= 16 && c0 >= 0 && c0 + C <= proj.size(1) && out.is_contiguous() && out.dim() == 2 &&
+                  out.size(0) == T && out.size(1) == C, "short_conv: shapes");
   TORCH_CHECK(state.is_contiguous() && state.dim() == 3 && state.size(1) == taps - 1 && state.size(2) == C,
-              "conv_silu: state [slots, taps - 1, C]");
-  HY_HIP(kafka_hy_conv_silu(f32, proj.data_ptr(), proj.stride(0), (int)c0, w.data_ptr(), b.data_ptr(), (int)C,
-                            (int)taps, tok_seg.data_ptr<int>(), seg.data_ptr<int>(), (int)seg.size(0),
-                            state.data_ptr(), out.data_ptr(), T, stream()));
+              "short_conv: state [slots, taps - 1, C]");
+  TORCH_CHECK(out.data_ptr() != proj.data_ptr(), "short_conv: out must not alias the input");
+  HY_HIP(kafka_hy_short_conv(f32, proj.data_ptr(), proj.stride(0), (int)c0, w.data_ptr(),
+                             b.has_value() ? b->data_ptr() : nullptr, (int)C, (int)taps, tok_seg.data_ptr<int>(),
+                             seg.data_ptr<int>(), (int)seg.size(0), state.data_ptr(), out.data_ptr(), T, (int)silu,
+                             (int)residual, stream()));
 }
 
 void ssm_scan(at::Tensor xbc, at::Tensor proj, int64_t dt_off, at::Tensor dt_bias, at::Tensor A_log, at::Tensor D,
@@ -387,7 +433,237 @@ void gated_norm(at::Tensor y, at::Tensor proj, at::Tensor w, int64_t groups, dou
                              (int)inner, (int)groups, (float)eps, out.data_ptr(), out.stride(0), T, stream()));
 }
 
+// ---- gated mixers ----------------------------------------------------------------------------------------------------
+void f32t(const at::Tensor& t, const char* name) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::kFloat, name, ": fp32 GPU tensor expected");
+}
+
+void rms_norm(at::Tensor x, at::Tensor w, double eps, at::Tensor out) {
+  rows2d(x, "x"); rows2d(out, "out"); f32t(x, "x");
+  const int f32 = act_f32(out);
+  same_act(f32, {&w});
+  const int64_t T = x.size(0), d = x.size(1);
+  vec(w, d, "w");
+  TORCH_CHECK(out.size(0) == T && out.size(1) == d, "rms_norm: out shape");
+  HY_HIP(kafka_hy_rms_norm(f32, x.data_ptr<float>(), x.stride(0), w.data_ptr(), (float)eps, out.data_ptr(),
+                           out.stride(0), (int)T, (int)d, stream()));
+}
+
+void kv_store(at::Tensor src, int64_t k_off, int64_t v_off, at::Tensor kc, at::Tensor vt, at::Tensor slots) {
+  rows2d(src, "src");
+  const int f32 = act_f32(src);
+  same_act(f32, {&kc, &vt});
+  const int64_t T = src.size(0);
+  TORCH_CHECK(kc.is_contiguous() && kc.dim() == 3 && kc.size(1) == 16, "kv_store: keys [pages, 16, Ck]");
+  TORCH_CHECK(vt.is_contiguous() && vt.dim() == 3 && vt.size(2) == 16 && vt.size(0) == kc.size(0),
+              "kv_store: values [pages, Cv, 16]");
+  const int64_t Ck = kc.size(2), Cv = vt.size(1);
+  TORCH_CHECK(k_off >= 0 && k_off + Ck <= src.size(1) && v_off >= 0 && v_off + Cv <= src.size(1), "kv_store: columns");
+  TORCH_CHECK(slots.is_cuda() && slots.scalar_type() == at::kLong && slots.is_contiguous() && slots.numel() == T,
+              "kv_store: slots int64 [T]");
+  HY_HIP(kafka_hy_kv_store(f32, src.data_ptr(), src.stride(0), (int)k_off, (int)v_off, (int)Ck, (int)Cv, kc.data_ptr(),
+                           vt.data_ptr(), slots.data_ptr<int64_t>(), T, stream()));
+}
+
+struct SigShape { int64_t T, D, Dv; int f32; };
+
+SigShape sig_check(const at::Tensor& q, int64_t q_off, const at::Tensor& kc, const at::Tensor& vt, const at::Tensor& bt,
+                   const at::Tensor& positions, int64_t H, int64_t G, const at::Tensor& r1, const at::Tensor& r2,
+                   const at::Tensor& pb, const at::Tensor& out) {
+  rows2d(q, "q"); rows2d(out, "out");
+  const int f32 = act_f32(q);
+  same_act(f32, {&kc, &vt, &out});
+  const int64_t T = q.size(0);
+  TORCH_CHECK(G >= 1 && H >= 1 && H % G == 0, "sigmoid_attn: heads");
+  TORCH_CHECK(kc.is_contiguous() && kc.dim() == 3 && kc.size(1) == 16 && kc.size(2) % G == 0,
+              "sigmoid_attn: keys [pages, 16, G D]");
+  TORCH_CHECK(vt.is_contiguous() && vt.dim() == 3 && vt.size(2) == 16 && vt.size(0) == kc.size(0) && vt.size(1) % G == 0,
+              "sigmoid_attn: values [pages, G Dv, 16]");
+  const int64_t D = kc.size(2) / G, Dv = vt.size(1) / G;
+  TORCH_CHECK(q_off >= 0 && q_off + H * D <= q.size(1), "sigmoid_attn: query columns");
+  TORCH_CHECK(out.size(0) == T && out.size(1) == H * Dv, "sigmoid_attn: out [T, H Dv]");
+  TORCH_CHECK(bt.is_cuda() && bt.scalar_type() == at::kInt && bt.dim() == 2 && bt.stride(1) == 1, "sigmoid_attn: bt");
+  TORCH_CHECK(positions.is_cuda() && positions.scalar_type() == at::kLong && positions.is_contiguous() &&
+                  positions.numel() == T, "sigmoid_attn: positions int64 [T]");
+  f32t(r1, "r1"); f32t(r2, "r2"); f32t(pb, "pb");
+  vec(r1, H, "r1"); vec(r2, H, "r2"); vec(pb, H, "pb");
+  return {T, D, Dv, f32};
+}
+
+void sigmoid_attn(at::Tensor q, int64_t q_off, at::Tensor kc, at::Tensor vt, at::Tensor bt, at::Tensor tok_seg,
+                  at::Tensor positions, int64_t H, int64_t G, double scale, double softcap, double t_coef,
+                  double t_every, at::Tensor r1, at::Tensor r2, at::Tensor pb, at::Tensor out) {
+  const SigShape s = sig_check(q, q_off, kc, vt, bt, positions, H, G, r1, r2, pb, out);
+  TORCH_CHECK(tok_seg.is_cuda() && tok_seg.scalar_type() == at::kInt && tok_seg.is_contiguous() &&
+                  tok_seg.numel() == s.T, "sigmoid_attn: tok_seg int32 [T]");
+  TORCH_CHECK(s.D <= kafka_hy_sigmoid_attn_max_d() && s.Dv <= kafka_hy_sigmoid_attn_max_dv(),
+              "sigmoid_attn: head sizes up to ", kafka_hy_sigmoid_attn_max_d(), " / ", kafka_hy_sigmoid_attn_max_dv());
+  TORCH_CHECK(t_coef == 0.0 || t_every > 0.0, "sigmoid_attn: temperature period");
+  HY_HIP(kafka_hy_sigmoid_attn(s.f32, q.data_ptr(), q.stride(0), (int)q_off, kc.data_ptr(), vt.data_ptr(),
+                               bt.data_ptr<int>(), (int)bt.stride(0), tok_seg.data_ptr<int>(),
+                               positions.data_ptr<int64_t>(), (int)H, (int)G, (int)s.D, (int)s.Dv, (float)scale,
+                               (float)softcap, (float)t_coef, t_every, r1.data_ptr<float>(), r2.data_ptr<float>(),
+                               pb.data_ptr<float>(), out.data_ptr(), out.stride(0), s.T, stream()));
+}
+
+void sigmoid_attn_mfma(at::Tensor q, int64_t q_off, at::Tensor kc, at::Tensor vt, at::Tensor bt, at::Tensor items,
+                       int64_t tile_tokens, at::Tensor positions, int64_t H, int64_t G, double scale, double softcap,
+                       double t_coef, double t_every, at::Tensor r1, at::Tensor r2, at::Tensor pb, at::Tensor out,
+                       int64_t nsplit, OptT po) {
+  const SigShape s = sig_check(q, q_off, kc, vt, bt, positions, H, G, r1, r2, pb, out);
+  TORCH_CHECK(!s.f32, "sigmoid_attn_mfma: bf16 only");
+  TORCH_CHECK(kafka_hy_sigmoid_attn_mfma_ok(16, (int)s.D, (int)s.Dv, (int)(H / G)), "sigmoid_attn_mfma: sizes");
+  TORCH_CHECK(q.stride(0) % 8 == 0 && q_off % 8 == 0 && (reinterpret_cast<uintptr_t>(q.data_ptr()) & 15) == 0,
+              "sigmoid_attn_mfma: query rows must be 16-byte aligned");
+  TORCH_CHECK(items.is_cuda() && items.scalar_type() == at::kInt && items.is_contiguous() && items.dim() == 2 &&
+                  items.size(1) == 4, "sigmoid_attn_mfma: items int32 [n, 4]");
+  TORCH_CHECK(tile_tokens >= 1 && tile_tokens * (H / G) <= 32 || (tile_tokens == 1 && H / G <= 32),
+              "sigmoid_attn_mfma: a tile holds at most 32 (token, head) rows");
+  TORCH_CHECK(t_coef == 0.0 || t_every > 0.0, "sigmoid_attn_mfma: temperature period");
+  float* pop = nullptr;
+  if (nsplit > 1) {
+    TORCH_CHECK(po.has_value() && po->is_cuda() && po->scalar_type() == at::kFloat && po->is_contiguous() &&
+                    po->numel() == nsplit * s.T * H * s.Dv, "sigmoid_attn_mfma: po fp32 [nsplit, T, H Dv]");
+    pop = po->data_ptr<float>();
+  }
+  HY_HIP(kafka_hy_sigmoid_attn_mfma(q.data_ptr(), q.stride(0), (int)q_off, kc.data_ptr(), vt.data_ptr(),
+                                    bt.data_ptr<int>(), (int)bt.stride(0), items.data_ptr<int>(), (int)items.size(0),
+                                    positions.data_ptr<int64_t>(), (int)H, (int)G, (int)s.D, (int)s.Dv, (float)scale,
+                                    (float)softcap, (float)t_coef, t_every, r1.data_ptr<float>(),
+                                    r2.data_ptr<float>(), pb.data_ptr<float>(), out.data_ptr(), out.stride(0),
+                                    (int)nsplit, pop, s.T, stream()));
+}
+
+void seg_only(const at::Tensor& seg) {
+  TORCH_CHECK(seg.is_cuda() && seg.scalar_type() == at::kInt && seg.is_contiguous() && seg.dim() == 2 &&
+                  seg.size(1) == 4, "seg: int32 [R, 4]");
+}
+
+void rglru_scan(at::Tensor gates, at::Tensor proj, at::Tensor u, at::Tensor rate, at::Tensor seg, at::Tensor state,
+                at::Tensor out, int64_t max_rows) {
+  rows2d(gates, "gates"); rows2d(proj, "proj"); rows2d(u, "u"); rows2d(out, "out");
+  f32t(gates, "gates"); f32t(rate, "rate"); f32t(state, "state");
+  const int f32 = act_f32(u);
+  same_act(f32, {&proj, &out});
+  const int64_t T = u.size(0), W = u.size(1);
+  vec(rate, W, "rate");
+  seg_only(seg);
+  TORCH_CHECK(gates.size(0) == T && gates.size(1) == 2 * W && proj.size(0) == T && proj.size(1) >= W &&
+                  out.size(0) == T && out.size(1) == W, "rglru_scan: shapes");
+  TORCH_CHECK(state.is_contiguous() && state.dim() == 2 && state.size(1) == W, "rglru_scan: state fp32 [slots, W]");
+  const int64_t R = seg.size(0), CH = kafka_hy_rglru_chunk();
+  if (max_rows > CH && R > 0) {
+    // long segments: the chunked form (the gates tensor is overwritten with the decays and inputs)
+    TORCH_CHECK(max_rows <= T, "rglru_scan: max_rows beyond the step's rows");
+    const int64_t nch = (max_rows + CH - 1) / CH;
+    auto ab = at::empty({R * nch * 2 * W}, gates.options());
+    HY_HIP(kafka_hy_rglru_scan_chunked(f32, gates.data_ptr<float>(), gates.stride(0), proj.data_ptr(), proj.stride(0),
+                                       u.data_ptr(), u.stride(0), rate.data_ptr<float>(), seg.data_ptr<int>(), (int)R,
+                                       (int)nch, ab.data_ptr<float>(), state.data_ptr<float>(), out.data_ptr(),
+                                       out.stride(0), T, (int)W, stream()));
+    return;
+  }
+  HY_HIP(kafka_hy_rglru_scan(f32, gates.data_ptr<float>(), gates.stride(0), proj.data_ptr(), proj.stride(0),
+                             u.data_ptr(), u.stride(0), rate.data_ptr<float>(), seg.data_ptr<int>(), (int)seg.size(0),
+                             state.data_ptr<float>(), out.data_ptr(), out.stride(0), (int)W, stream()));
+}
+
+void mlstm_scan(at::Tensor qkv, at::Tensor gates, int64_t H, int64_t D, int64_t Dv, double cap, at::Tensor seg,
+                at::Tensor S, at::Tensor nrm, at::Tensor mx, at::Tensor out) {
+  rows2d(qkv, "qkv"); rows2d(gates, "gates"); rows2d(out, "out");
+  f32t(gates, "gates"); f32t(S, "S"); f32t(nrm, "n"); f32t(mx, "m"); f32t(out, "out");
+  const int f32 = act_f32(qkv);
+  const int64_t T = qkv.size(0);
+  seg_only(seg);
+  TORCH_CHECK(H >= 1 && D >= 1 && Dv >= 1 && D <= kafka_hy_mlstm_max_d(), "mlstm_scan: head sizes (dim up to ",
+              kafka_hy_mlstm_max_d(), ")");
+  TORCH_CHECK(cap > 0.0, "mlstm_scan: gate cap");
+  TORCH_CHECK(qkv.size(1) >= H * (2 * D + Dv) && gates.size(0) == T && gates.size(1) == 2 * H && out.size(0) == T &&
+                  out.size(1) == H * Dv, "mlstm_scan: shapes");
+  const int64_t slots = S.size(0);
+  TORCH_CHECK(S.is_contiguous() && S.dim() == 4 && S.size(1) == H && S.size(2) == D && S.size(3) == Dv &&
+                  nrm.is_contiguous() && nrm.dim() == 3 && nrm.size(0) == slots && nrm.size(1) == H &&
+                  nrm.size(2) == D && mx.is_contiguous() && mx.dim() == 2 && mx.size(0) == slots && mx.size(1) == H,
+              "mlstm_scan: state S [slots, H, D, Dv], n [slots, H, D], m [slots, H]");
+  HY_HIP(kafka_hy_mlstm_scan(f32, qkv.data_ptr(), qkv.stride(0), gates.data_ptr<float>(), gates.stride(0), (int)H,
+                             (int)D, (int)Dv, (float)cap, seg.data_ptr<int>(), (int)seg.size(0), S.data_ptr<float>(),
+                             nrm.data_ptr<float>(), mx.data_ptr<float>(), out.data_ptr<float>(), out.stride(0),
+                             stream()));
+}
+
+void head_norm_gate(at::Tensor o, at::Tensor w, at::Tensor g, int64_t g_off, int64_t H, double eps, at::Tensor out) {
+  rows2d(o, "o"); rows2d(g, "g"); rows2d(out, "out"); f32t(o, "o");
+  const int f32 = act_f32(out);
+  same_act(f32, {&w, &g});
+  const int64_t T = o.size(0), n = o.size(1);
+  vec(w, n, "w");
+  TORCH_CHECK(H >= 1 && n % H == 0 && g.size(0) == T && g_off >= 0 && g_off + n <= g.size(1) && out.size(0) == T &&
+                  out.size(1) == n, "head_norm_gate: shapes");
+  HY_HIP(kafka_hy_head_norm_gate(f32, o.data_ptr<float>(), o.stride(0), w.data_ptr(), g.data_ptr(), g.stride(0),
+                                 (int)g_off, (int)H, (int)(n / H), (float)eps, out.data_ptr(), out.stride(0), T,
+                                 stream()));
+}
+
+void moe_topk(at::Tensor logits, at::Tensor tw, at::Tensor te) {
+  rows2d(logits, "logits"); f32t(logits, "logits"); f32t(tw, "weights");
+  const int64_t T = logits.size(0), E = logits.size(1);
+  TORCH_CHECK(tw.is_contiguous() && tw.dim() == 2 && tw.size(0) == T && te.is_cuda() && te.is_contiguous() &&
+                  te.scalar_type() == at::kInt && te.sizes() == tw.sizes(), "moe_topk: outputs [T, k]");
+  const int64_t k = tw.size(1);
+  TORCH_CHECK(E <= kafka_hy_router_max_e() && k >= 1 && k <= kafka_hy_router_max_k() && k <= E,
+              "moe_topk: up to ", kafka_hy_router_max_e(), " experts, ", kafka_hy_router_max_k(), " per row");
+  HY_HIP(kafka_hy_moe_topk(logits.data_ptr<float>(), logits.stride(0), (int)E, (int)k, tw.data_ptr<float>(),
+                           te.data_ptr<int>(), T, stream()));
+}
+
+void moe_rows(at::Tensor h, at::Tensor wgu, at::Tensor wd, at::Tensor tw, at::Tensor te, at::Tensor a, at::Tensor out) {
+  rows2d(h, "h"); rows2d(out, "out"); f32t(out, "out"); f32t(tw, "weights");
+  const int f32 = act_f32(h);
+  same_act(f32, {&wgu, &wd, &a});
+  const int64_t T = h.size(0), d = h.size(1);
+  TORCH_CHECK(wd.is_contiguous() && wd.dim() == 3 && wd.size(1) == d, "moe_rows: w_down [E, d, F]");
+  const int64_t E = wd.size(0), F = wd.size(2);
+  TORCH_CHECK(wgu.is_contiguous() && wgu.dim() == 3 && wgu.size(0) == E && wgu.size(1) == 2 * F && wgu.size(2) == d,
+              "moe_rows: w_gu [E, 2 F, d]");
+  TORCH_CHECK(tw.is_contiguous() && tw.dim() == 2 && tw.size(0) == T && te.is_cuda() && te.is_contiguous() &&
+                  te.scalar_type() == at::kInt && te.sizes() == tw.sizes(), "moe_rows: routing [T, k]");
+  const int64_t k = tw.size(1);
+  TORCH_CHECK(a.is_contiguous() && a.numel() == T * k * F, "moe_rows: scratch [T k, F]");
+  TORCH_CHECK(out.size(0) == T && out.size(1) == d, "moe_rows: out [T, d]");
+  TORCH_CHECK(d <= kafka_hy_moe_rows_max_d() && F <= kafka_hy_moe_rows_max_d(), "moe_rows: row sizes up to ",
+              kafka_hy_moe_rows_max_d());
+  // expert ids index the weight stacks on the device: the router kernel writes ids in [0, E) only
+  HY_HIP(kafka_hy_moe_rows(f32, h.data_ptr(), h.stride(0), wgu.data_ptr(), wd.data_ptr(), tw.data_ptr<float>(),
+                           te.data_ptr<int>(), (int)d, (int)F, (int)k, a.data_ptr(), out.data_ptr<float>(),
+                           out.stride(0), T, stream()));
+}
+
+void add2(at::Tensor x, at::Tensor y1, OptT y2, OptT w, double eps, OptT out) {
+  rows2d(x, "x"); rows2d(y1, "y1"); f32t(x, "x");
+  const int f32 = act_f32(y1);
+  const int64_t T = x.size(0), d = x.size(1);
+  TORCH_CHECK(y1.size(0) == T && y1.size(1) == d, "add2: y1 shape");
+  const void* p2 = nullptr; int64_t s2 = 0; int y2f = 0;
+  if (y2.has_value()) {
+    rows2d(*y2, "y2");
+    TORCH_CHECK(y2->size(0) == T && y2->size(1) == d, "add2: y2 shape");
+    y2f = y2->scalar_type() == at::kFloat;
+    TORCH_CHECK(y2f || act_f32(*y2) == f32, "add2: y2 is fp32 or of y1's dtype");
+    p2 = y2->data_ptr(); s2 = y2->stride(0);
+  }
+  const void* wp = nullptr; void* op = nullptr; int64_t os = 0;
+  if (w.has_value()) {
+    TORCH_CHECK(out.has_value(), "add2: a norm weight needs an output");
+    same_act(f32, {&*w, &*out}); vec(*w, d, "w"); rows2d(*out, "out");
+    TORCH_CHECK(out->size(0) == T && out->size(1) == d && x.stride(0) >= d, "add2: out shape");
+    wp = w->data_ptr(); op = out->data_ptr(); os = out->stride(0);
+  }
+  HY_HIP(kafka_hy_add2(f32, x.data_ptr<float>(), x.stride(0), y1.data_ptr(), y1.stride(0), p2, s2, y2f, T, (int)d, wp,
+                       (float)eps, op, os, stream()));
+}
+
 }  // namespace
+
 
 void kafka_bind_hybrid(pybind11::module_& m) {
   namespace py = pybind11;
@@ -410,9 +686,26 @@ void kafka_bind_hybrid(pybind11::module_& m) {
   m.def("hy_latent_mfma_ok", [](int page, int R, int rd) { return kafka_hy_latent_mfma_ok(page, R, rd) != 0; });
   m.def("hy_sigmoid_mul", &sigmoid_mul);
   m.def("hy_latent_attn", &latent_attn);
-  m.def("hy_conv_silu", &conv_silu);
+  m.def("hy_short_conv", &short_conv);
   m.def("hy_ssm_scan", &ssm_scan);
   m.def("hy_ssm_combine", &ssm_combine);
   m.def("hy_gated_norm", &gated_norm);
   m.def("hy_scan_groups", [](int P, int N) { return kafka_hy_scan_groups(P, N); });
+  m.def("hy_rms_norm", &rms_norm);
+  m.def("hy_kv_store", &kv_store);
+  m.def("hy_sigmoid_attn", &sigmoid_attn);
+  m.def("hy_rglru_scan", &rglru_scan, py::arg("gates"), py::arg("proj"), py::arg("u"), py::arg("rate"), py::arg("seg"),
+        py::arg("state"), py::arg("out"), py::arg("max_rows") = 0);
+  m.def("hy_mlstm_scan", &mlstm_scan);
+  m.def("hy_head_norm_gate", &head_norm_gate);
+  m.def("hy_moe_topk", &moe_topk);
+  m.def("hy_moe_rows", &moe_rows);
+  m.def("hy_add2", &add2, py::arg("x"), py::arg("y1"), py::arg("y2") = py::none(), py::arg("w") = py::none(),
+        py::arg("eps") = 0.0, py::arg("out") = py::none());
+  m.def("hy_sigmoid_attn_mfma_ok",
+        [](int page, int D, int Dv, int rep) { return kafka_hy_sigmoid_attn_mfma_ok(page, D, Dv, rep) != 0; });
+  m.def("hy_sigmoid_attn_mfma", &sigmoid_attn_mfma, py::arg("q"), py::arg("q_off"), py::arg("kc"), py::arg("vt"),
+        py::arg("bt"), py::arg("items"), py::arg("tile_tokens"), py::arg("positions"), py::arg("H"), py::arg("G"),
+        py::arg("scale"), py::arg("softcap"), py::arg("t_coef"), py::arg("t_every"), py::arg("r1"), py::arg("r2"),
+        py::arg("pb"), py::arg("out"), py::arg("nsplit") = 1, py::arg("po") = py::none());
 }

@@ -52,8 +52,9 @@ __global__ __launch_bounds__(MOE_NT) void moe_route_kernel(const bf16* __restric
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int per = (T + MOE_NT - 1) / MOE_NT;  // tokens owned by this thread: [t0, t1)
   const int t0 = min(T, tid * per), t1 = min(T, t0 + per);
-  // ---- phase 1: softmax + top-k + renormalise for the owned tokens
-  for (int t = t0; t < t1; ++t) {
+  // ---- phase 1: softmax + top-k + renormalise for the owned tokens (logits == nullptr: the caller has routed -
+  // topk_w / topk_e are inputs, any number of experts and choices - and only the sort below runs)
+  for (int t = t0; logits != nullptr && t < t1; ++t) {
     float p[MOE_MAXE];
     float m = -INFINITY;
     for (int e = 0; e < E; ++e) {
@@ -256,7 +257,7 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(const bf16* __restric
 extern "C" hipError_t kafka_launch_moe_route(const bf16* logits, int64_t ld, int T, int E, int K, int BM,
                                             float* topk_w, int* topk_e, int* perm_tok, float* perm_w,
                                             int* expert_off, int* tile_off, hipStream_t st) {
-  if (E > MOE_MAXE || K > MOE_MAXK || K > E) return hipErrorInvalidValue;
+  if (K > E || K < 1 || (logits != nullptr && (E > MOE_MAXE || K > MOE_MAXK))) return hipErrorInvalidValue;
   moe_route_kernel<<<1, MOE_NT, 0, st>>>(logits, ld, T, E, K, BM, topk_w, topk_e, perm_tok, perm_w, expert_off,
                                          tile_off);
   return hipGetLastError();

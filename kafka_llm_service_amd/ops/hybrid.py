@@ -12,7 +12,7 @@ import torch
 from . import hybrid_reference as ref
 from ._ext import ext
 
-SCAN_MAX_TAPS = 8
+SCAN_MAX_TAPS = 16
 
 
 def _gpu(t: torch.Tensor) -> bool:
@@ -149,12 +149,21 @@ def sigmoid_mul(a, g, out) -> None:
 def conv_silu(proj, c0: int, w, b, tok_seg, seg, state, out) -> None:
     """Causal per-channel convolution + silu over columns [c0, c0 + C) of ``proj``; ``state`` [slots, taps - 1, C]
     holds each sequence's last raw inputs and is advanced."""
+    short_conv(proj, c0, w, b, tok_seg, seg, state, out, act="silu")
+
+
+def short_conv(u, c0: int, w, b, tok_seg, seg, state, out, act: str = "none", residual: bool = False) -> None:
+    """out_t = act(b + sum_k w[:, k] u_(t - taps + 1 + k)) (+ u_t with ``residual``) per channel of columns
+    [c0, c0 + C) of ``u``, zeros before a sequence's start; ``b`` may be None, ``act`` is "none" or "silu".
+    ``state`` [slots, taps - 1, C] holds each sequence's last inputs and is advanced (taps = 1: no state)."""
     if w.shape[1] > SCAN_MAX_TAPS:
         raise ValueError(f"short convolution of {w.shape[1]} taps (at most {SCAN_MAX_TAPS})")
-    if _gpu(proj):
-        ext().hy_conv_silu(proj, int(c0), w, b, tok_seg, seg, state, out)
+    if act not in ("none", "silu"):
+        raise ValueError(f"short convolution: unknown activation {act!r}")
+    if _gpu(u):
+        ext().hy_short_conv(u, int(c0), w, b, tok_seg, seg, state, out, act == "silu", bool(residual))
     else:
-        ref.conv_silu(proj, c0, w, b, tok_seg, seg, state, out)
+        ref.short_conv(u, c0, w, b, tok_seg, seg, state, out, act, residual)
 
 
 def ssm_scan(xbc, proj, dt_off: int, dt_bias, A_log, D, heads, P, N, G, tok_seg, seg, state, y) -> None:
@@ -215,3 +224,188 @@ def gated_norm(y, proj, w, groups: int, eps, out) -> None:
         ext().hy_gated_norm(y, proj, w, int(groups), float(eps), out)
     else:
         ref.gated_norm(y, proj, w, groups, eps, out)
+
+
+# ---- gated mixers: sigmoid attention, real-gated linear recurrence, matrix memory, routed experts --------------------
+def rms_norm(x, w, eps, out) -> None:
+    """out = x / sqrt(mean(x^2) + eps) * w over rows of the fp32 stream."""
+    if _gpu(x):
+        ext().hy_rms_norm(x, w, float(eps), out)
+    else:
+        ref.rms_norm(x, w, eps, out)
+
+
+def kv_store(src, k_off: int, v_off: int, k_cache, v_cache_t, slot_mapping) -> None:
+    """Row t's key columns [k_off, k_off + Ck) -> k_cache [pages, page, Ck] at its slot, its value columns
+    [v_off, v_off + Cv) -> v_cache_t [pages, Cv, page] (every page transposed: a channel's tokens are consecutive,
+    the layout the value product of the attention kernels reads)."""
+    if _gpu(src):
+        ext().hy_kv_store(src, int(k_off), int(v_off), k_cache, v_cache_t, slot_mapping)
+    else:
+        ref.kv_store(src, k_off, v_off, k_cache, v_cache_t, slot_mapping)
+
+
+SIG_TILE_ROWS = 32     # query rows ((token, head) pairs of one key/value head) of a matrix-core attention tile
+
+
+def sig_tile_tokens(heads: int, kv_heads: int) -> int:
+    """Tokens per tile of the matrix-core sigmoid attention: as many whole tokens (all query heads of one key/value
+    head) as fit 32 rows, at least one."""
+    return max(1, SIG_TILE_ROWS // max(1, heads // kv_heads))
+
+
+def sigmoid_attn_mfma_ok(q, k_cache, v_cache_t, H: int, G: int) -> bool:
+    """bf16 GPU tensors of sizes the matrix-core kernel takes (16-token pages, key size a multiple of 16, sizes up
+    to 256, at most 32 query heads per key/value head, 16-byte aligned query rows)."""
+    if not (q.is_cuda and q.dtype == torch.bfloat16):
+        return False
+    if q.stride(0) % 8 or q.data_ptr() % 16:  # query rows are read in 16-byte pieces
+        return False
+    return bool(ext().hy_sigmoid_attn_mfma_ok(k_cache.shape[1], k_cache.shape[2] // G, v_cache_t.shape[1] // G,
+                                              H // G))
+
+
+def sig_splits(wgs: int, max_keys: int) -> int:
+    """Key-range splits of a matrix-core sigmoid attention launch: few workgroups (a decode step has one tile per
+    sequence and key/value head) against long contexts are dealt over more, each at least two 128-key blocks long; the
+    partial sums are added in order by a second launch."""
+    blocks = -(-max_keys // 128)
+    if wgs >= ATTN_SPLIT_WGS // 2 or blocks < 4:
+        return 1
+    return max(1, min(ATTN_SPLIT_MAX, ATTN_SPLIT_WGS // max(1, wgs), blocks // 2))
+
+
+def sigmoid_attn(q, q_off: int, k_cache, v_cache_t, block_tables, tok_seg, positions, H: int, G: int, scale: float,
+                 softcap: float, t_coef: float, t_every: float, r1, r2, pb, out, tiles=None, max_keys: int = 0) -> None:
+    """Causal attention with sigmoid weights (no softmax, no normalisation over keys). For row t at position p, head h
+    (key/value head h // (H / G)) and every key j <= p:
+        s = (q . k_j) scale (1 + t_coef ln(floor((p + 1) / t_every) + 1));  s = softcap tanh(s / softcap) if softcap;
+        out = sum_j sigmoid(s - r1[h] ln(1 + r2[h] (p - j)) + pb[h]) v_j.
+    q rows start at column ``q_off`` of ``q``; out [T, H Dv]. Scores, biases and weights are fp32. With ``tiles``
+    (int32 [n, 4] = (first row, tokens, segment, 0), at most ``sig_tile_tokens`` tokens of one segment each) and
+    sizes it takes, bf16 runs on the matrix cores; else one wave per (row, head) on the vector units. ``max_keys``
+    (the step's longest context) lets a launch of few tiles split its key ranges over more workgroups."""
+    if _gpu(q):
+        if tiles is not None and q_off % 8 == 0 and sigmoid_attn_mfma_ok(q, k_cache, v_cache_t, H, G):
+            ns = sig_splits(tiles.shape[0] * G, max_keys) if max_keys else 1
+            po = None
+            if ns > 1:
+                po = torch.empty(ns, q.shape[0], out.shape[1], dtype=torch.float32, device=q.device)
+            ext().hy_sigmoid_attn_mfma(q, int(q_off), k_cache, v_cache_t, block_tables, tiles,
+                                       sig_tile_tokens(H, G), positions, int(H), int(G), float(scale), float(softcap),
+                                       float(t_coef), float(t_every), r1, r2, pb, out, ns, po)
+        else:
+            ext().hy_sigmoid_attn(q, int(q_off), k_cache, v_cache_t, block_tables, tok_seg, positions, int(H), int(G),
+                                  float(scale), float(softcap), float(t_coef), float(t_every), r1, r2, pb, out)
+    else:
+        ref.sigmoid_attn(q, q_off, k_cache, v_cache_t, block_tables, tok_seg, positions, H, G, scale, softcap, t_coef,
+                         t_every, r1, r2, pb, out)
+
+
+def rglru_scan(gates, proj, u, rate, tok_seg, seg, state, out, max_rows: int = 0) -> None:
+    """The real-gated linear recurrent unit over a step's segments. gates fp32 [T, 2 W] = pre-activations of the
+    recurrence gate | the input gate (biases included), proj [T, >= W] whose first W columns are the raw gelu branch,
+    u [T, W] the convolved branch, rate fp32 [W] (= -c softplus(lambda)):
+        a = exp(rate sigmoid(g_r)),  S <- a S + sqrt(1 - a^2) sigmoid(g_i) u,  out = S gelu_tanh(branch).
+    state fp32 [slots, W], zero before a sequence's first token (the slot is then written, not read). ``max_rows``:
+    an upper bound of the longest segment's rows, when the caller knows one: steps with segments of more than 64 rows
+    run in chunks (everything but the multiply-adds in parallel over rows, the chunks' entry states carried in
+    order; ``gates`` is then overwritten), which re-associates the sums - fp32 rounding only."""
+    if _gpu(u):
+        ext().hy_rglru_scan(gates, proj, u, rate, seg, state, out, int(max_rows))
+    else:
+        ref.rglru_scan(gates, proj, u, rate, tok_seg, seg, state, out)
+
+
+def mlstm_scan(qkv, gates, H: int, D: int, Dv: int, cap: float, tok_seg, seg, S, nrm, mx, out) -> None:
+    """The matrix-memory recurrence (mLSTM) over a step's segments. qkv [T, >= H (2 D + Dv)] = q | k | v heads,
+    gates fp32 [T, 2 H] = raw input | forget gate (biases included). Per head, with i = cap tanh(g_i / cap),
+    f = logsigmoid(cap tanh(g_f / cap)), q' = q D^(-1/2):
+        m' = max(f + m, i);  S <- e^(f + m - m') S + e^(i - m') k v^T;  n <- e^(f + m - m') n + e^(i - m') k;
+        out = S^T q' / (max(|n . q'|, e^(-m')) + 1e-6).
+    State per slot, all fp32 and all zero (m too) before a sequence's first token: S [slots, H, D, Dv],
+    nrm [slots, H, D], mx [slots, H]. out fp32 [T, H Dv]."""
+    if _gpu(qkv):
+        ext().hy_mlstm_scan(qkv, gates, int(H), int(D), int(Dv), float(cap), seg, S, nrm, mx, out)
+    else:
+        ref.mlstm_scan(qkv, gates, H, D, Dv, cap, tok_seg, seg, S, nrm, mx, out)
+
+
+def head_norm_gate(o, w, g, g_off: int, H: int, eps, out) -> None:
+    """out = o / rms_per_head(o) * w * sigmoid(g[:, g_off : g_off + H Dv]) for o fp32 [T, H Dv]."""
+    if _gpu(o):
+        ext().hy_head_norm_gate(o, w, g, int(g_off), int(H), float(eps), out)
+    else:
+        ref.head_norm_gate(o, w, g, g_off, H, eps, out)
+
+
+def moe_router(h, w, b, k: int):
+    """Router of a routed feed-forward: fp32 logits h W^T + b (W, b fp32), the k largest per row (ties: the lower
+    index) and a softmax over those k. Returns (weights fp32 [T, k], experts int32 [T, k])."""
+    T = h.shape[0]
+    tw = torch.empty(T, k, dtype=torch.float32, device=h.device)
+    te = torch.empty(T, k, dtype=torch.int32, device=h.device)
+    if k > w.shape[0]:
+        raise ValueError("router: more experts per token than experts")
+    if _gpu(h):
+        # logits as one fp32 matrix product (full-precision fp32: PyTorch's default for fp32 operands, and the engine
+        # switches reduced-precision matrix modes off explicitly for fp32 models), then the top-k kernel
+        ext().hy_moe_topk(torch.addmm(b, h.float(), w.t()), tw, te)
+    else:
+        ref.moe_router(h, w, b, k, tw, te)
+    return tw, te
+
+
+def moe_rows(h, w_gu, w_down, topk_w, topk_e, out) -> None:
+    """Routed experts evaluated per (row, chosen expert) pair, any sizes and both dtypes:
+    out[t] = sum_j topk_w[t, j] W_down[e_tj] (silu(W_gate[e_tj] h_t) * W_up[e_tj] h_t) with w_gu [E, 2 F, d] = gate
+    rows then up rows and w_down [E, d, F]; the pairs of a row are summed in order j = 0, 1, ... (fp32)."""
+    if _gpu(h):
+        T, k = topk_e.shape
+        a = torch.empty(T * k, w_down.shape[2], dtype=h.dtype, device=h.device)
+        ext().hy_moe_rows(h, w_gu, w_down, topk_w, topk_e, a, out)
+    else:
+        ref.moe_rows(h, w_gu, w_down, topk_w, topk_e, out)
+
+
+MOE_STREAM_MAX_T = 640  # steps of up to this many rows run tiled expert weights on the grouped streaming kernel
+
+
+def moe_grouped_ok(h, w_gu, w_down) -> bool:
+    """bf16 GPU tensors of sizes the expert-sorted matrix-core kernels take (ops.grouped_gemm)."""
+    E, F2, d = w_gu.shape
+    return bool(h.is_cuda and h.dtype == torch.bfloat16 and F2 % 128 == 0 and d % 128 == 0 and (F2 // 2) % 64 == 0 and
+                h.stride(0) % 8 == 0)
+
+
+def moe_experts(h, w_gu, w_down, topk_w, topk_e, out, w_gu_t=None, w_down_t=None) -> None:
+    """out (fp32 [T, d]) = the routed experts' weighted sum for every row. Sizes the framework's expert-sorted
+    matrix-core kernels take (bf16) go through them - entries sorted by expert (``ops.moe_sort``), gate/up GEMM on
+    gathered rows, silu * up, down GEMM with the weighted combine in its epilogue (fp32 adds, two entries per row
+    commute), or the grouped weight-streaming kernels when tiled expert weights are given and the step is small -
+    everything else is evaluated per (row, expert) pair by ``moe_rows``."""
+    from kafka_llm_service_amd import ops
+
+    T = h.shape[0]
+    if T and moe_grouped_ok(h, w_gu, w_down):
+        r = ops.moe_sort(topk_w, topk_e, w_gu.shape[0])
+        out.zero_()
+        if w_gu_t is not None and w_down_t is not None and T <= MOE_STREAM_MAX_T:
+            a = ops.grouped_stream_glu(h, w_gu_t, r)
+            ops.grouped_stream_combine(a, w_down_t, r, T, out)
+        else:
+            a = ops.silu_mul(ops.grouped_gemm(h, w_gu, r, gather=True))
+            ops.grouped_gemm(a, w_down, r, gather=False, combine_out=out)
+    else:
+        moe_rows(h, w_gu, w_down, topk_w, topk_e, out)
+
+
+def add2(x, y1, y2=None, norm_w=None, eps=0.0, out=None) -> None:
+    """x += y1 (+ y2) on the fp32 stream, the sublayer outputs summed in fp32 first; with ``norm_w`` also
+    out = rms_norm(new x) * norm_w in the same pass over the row (the next layer's norm)."""
+    if _gpu(x):
+        ext().hy_add2(x, y1, y2, norm_w, float(eps), out)
+    else:
+        ref.add2(x, y1, y2)
+        if norm_w is not None:
+            ref.rms_norm(x, norm_w, eps, out)

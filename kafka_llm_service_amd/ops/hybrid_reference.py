@@ -152,3 +152,147 @@ def gated_norm(y, proj, w, groups, eps, out):
     v = v.view(T, groups, inner // groups)
     v = v * torch.rsqrt((v * v).mean(-1, keepdim=True) + eps)
     out.copy_(v.reshape(T, inner) * w.float())
+
+
+# ---- gated mixers: sigmoid attention, real-gated linear recurrence, matrix memory, routed experts --------------------
+def rms_norm(x, w, eps, out):
+    v = x.float()
+    out.copy_(v * torch.rsqrt((v * v).mean(-1, keepdim=True) + eps) * w.float())
+
+
+def short_conv(u, c0, w, b, tok_seg, seg, state, out, act="none", residual=False):
+    """Causal per-channel convolution over columns [c0, c0 + C) of ``u``: out_t = act(b + sum_k w[:, k] u_(t - taps + 1
+    + k)) (+ u_t with ``residual``); ``state`` [slots, taps - 1, C] holds each sequence's last inputs and is advanced."""
+    C, taps = w.shape
+    x = u[:, c0:c0 + C].float()
+    for q0, n, p0, slot in seg.tolist():
+        hist = state[slot].float() if p0 > 0 and taps > 1 else torch.zeros(taps - 1, C)
+        full = torch.cat([hist, x[q0:q0 + n]], 0)
+        acc = b.float().expand(n, C).clone() if b is not None else torch.zeros(n, C)
+        for k in range(taps):
+            acc = acc + full[k:k + n] * w[:, k].float()
+        if act == "silu":
+            acc = F.silu(acc)
+        if residual:
+            acc = acc + x[q0:q0 + n]
+        out[q0:q0 + n] = acc.to(out.dtype)
+        if taps > 1:
+            state[slot] = full[n:].to(state.dtype)
+
+
+def kv_store(src, k_off, v_off, k_cache, v_cache_t, slot_mapping):
+    """Row t's key columns -> k_cache [pages, page, Ck] at its slot; its value columns -> v_cache_t [pages, Cv, page]
+    (each page transposed: a channel's 16 tokens are consecutive)."""
+    page, Ck = k_cache.shape[1], k_cache.shape[2]
+    Cv = v_cache_t.shape[1]
+    ok = slot_mapping >= 0
+    sl = slot_mapping[ok].long()
+    k_cache.view(-1, Ck)[sl] = src[ok][:, k_off:k_off + Ck].to(k_cache.dtype)
+    v_cache_t[sl // page, :, sl % page] = src[ok][:, v_off:v_off + Cv].to(v_cache_t.dtype)
+
+
+def sigmoid_attn(q, q_off, k_cache, v_cache_t, block_tables, tok_seg, positions, H, G, scale, softcap, t_coef,
+                 t_every, r1, r2, pb, out):
+    """q rows [T, >= q_off + H D]; out [T, H Dv] = sum over keys j <= position of
+    sigmoid(cap(q . k_j scale temp) - r1 ln(1 + r2 (position - j)) + pb) v_j per head, not normalised."""
+    T = q.shape[0]
+    page, D = k_cache.shape[1], k_cache.shape[2] // G
+    Dv = v_cache_t.shape[1] // G
+    for t in range(T):
+        r, p = int(tok_seg[t]), int(positions[t])
+        n = p + 1
+        pages = block_tables[r, :(n + page - 1) // page].long()
+        k = k_cache[pages].reshape(-1, G, D)[:n].float()                       # [n, G, D]
+        v = v_cache_t[pages].permute(0, 2, 1).reshape(-1, G, Dv)[:n].float()   # [n, G, Dv]
+        temp = 1.0 + t_coef * math.log(math.floor((p + 1) / t_every) + 1.0) if t_coef else 1.0
+        dist = (p - torch.arange(n)).float()
+        qt = q[t, q_off:q_off + H * D].float().view(H, D)
+        for h in range(H):
+            g = h // (H // G)
+            s = (k[:, g] @ qt[h]) * (scale * temp)
+            if softcap:
+                s = softcap * torch.tanh(s / softcap)
+            s = s - r1[h] * torch.log1p(r2[h] * dist) + pb[h]
+            out[t, h * Dv:(h + 1) * Dv] = (torch.sigmoid(s) @ v[:, g]).to(out.dtype)
+
+
+def rglru_scan(gates, proj, u, rate, tok_seg, seg, state, out):
+    """gates fp32 [T, 2 W] = pre-activations of the recurrence gate | the input gate (biases included), proj [T, >= W]
+    whose first W columns are the raw gelu branch, u [T, W] the convolved branch, rate fp32 [W] = -8 softplus(lam):
+    a = exp(rate sigmoid(g_r)), S <- a S + sqrt(1 - a^2) sigmoid(g_i) u, out = S gelu(branch); state fp32 [slots, W]."""
+    Wd = u.shape[1]
+    la = rate.float() * torch.sigmoid(gates[:, :Wd].float())
+    a = torch.exp(la)
+    inp = torch.sqrt(-torch.expm1(2.0 * la)) * torch.sigmoid(gates[:, Wd:].float()) * u.float()
+    y = gelu_tanh(proj[:, :Wd].float())
+    for q0, n, p0, slot in seg.tolist():
+        S = state[slot].clone() if p0 > 0 else torch.zeros(Wd)
+        for t in range(q0, q0 + n):
+            S = a[t] * S + inp[t]
+            out[t] = (S * y[t]).to(out.dtype)
+        state[slot] = S
+
+
+def mlstm_scan(qkv, gates, H, D, Dv, cap, tok_seg, seg, S, nrm, mx, out):
+    """qkv [T, >= H (2 D + Dv)] = q | k | v heads (q still unscaled), gates fp32 [T, 2 H] = raw input | forget gate
+    (biases included). Per head, with i = cap tanh(g_i / cap), f = logsigmoid(cap tanh(g_f / cap)):
+    m' = max(f + m, i), S <- e^(f + m - m') S + e^(i - m') k v^T, n likewise with k,
+    out = S^T q' / (max(|n . q'|, e^(-m')) + 1e-6), q' = q D^(-1/2). State per slot: S [H, D, Dv], n [H, D], m [H],
+    all fp32, zero (m too) before a sequence's first token. out fp32 [T, H Dv]."""
+    for q0, n, p0, slot in seg.tolist():
+        if p0 > 0:
+            Ss, ns, ms = S[slot].clone(), nrm[slot].clone(), mx[slot].clone()
+        else:
+            Ss, ns, ms = torch.zeros(H, D, Dv), torch.zeros(H, D), torch.zeros(H)
+        for t in range(q0, q0 + n):
+            q = qkv[t, :H * D].float().view(H, D) * D ** -0.5
+            k = qkv[t, H * D:2 * H * D].float().view(H, D)
+            v = qkv[t, 2 * H * D:2 * H * D + H * Dv].float().view(H, Dv)
+            ig = cap * torch.tanh(gates[t, :H].float() / cap)
+            fg = F.logsigmoid(cap * torch.tanh(gates[t, H:].float() / cap))
+            m_new = torch.maximum(fg + ms, ig)
+            dec, gain = torch.exp(fg + ms - m_new), torch.exp(ig - m_new)
+            Ss = dec[:, None, None] * Ss + gain[:, None, None] * k[:, :, None] * v[:, None, :]
+            ns = dec[:, None] * ns + gain[:, None] * k
+            ms = m_new
+            num = torch.einsum("hdv,hd->hv", Ss, q)
+            den = torch.maximum((ns * q).sum(-1).abs(), torch.exp(-ms)) + 1e-6
+            out[t] = (num / den[:, None]).reshape(-1)
+        S[slot], nrm[slot], mx[slot] = Ss, ns, ms
+
+
+def head_norm_gate(o, w, g, g_off, H, eps, out):
+    """out = unit_rms_per_head(o) * w * sigmoid(g[:, g_off : g_off + H Dv]) (o fp32 [T, H Dv])."""
+    T, n = o.shape
+    v = o.float().view(T, H, n // H)
+    v = v * torch.rsqrt((v * v).mean(-1, keepdim=True) + eps)
+    out.copy_(v.reshape(T, n) * w.float() * torch.sigmoid(g[:, g_off:g_off + n].float()))
+
+
+def moe_router(h, w, b, k, topk_w, topk_e):
+    """fp32 logits h W^T + b; the k largest (ties: the lower index first) and a softmax over those k."""
+    z = h.float() @ w.float().T + b.float()
+    val, idx = torch.sort(z, dim=-1, descending=True, stable=True)
+    topk_e.copy_(idx[:, :k])
+    topk_w.copy_(torch.softmax(val[:, :k], -1))
+
+
+def moe_rows(h, w_gu, w_down, topk_w, topk_e, out):
+    """out[t] = sum_j topk_w[t, j] W_down[e] (silu(W_gate[e] h_t) * W_up[e] h_t), e = topk_e[t, j]; w_gu [E, 2 F, d]
+    = gate rows then up rows, w_down [E, d, F]; out in the activation dtype."""
+    T, k = topk_e.shape
+    Fh = w_down.shape[2]
+    hf = h.float()
+    acc = torch.zeros(T, w_down.shape[1])
+    for j in range(k):
+        e = topk_e[:, j].long()
+        gu = torch.einsum("tfd,td->tf", w_gu[e].float(), hf)
+        a = (F.silu(gu[:, :Fh]) * gu[:, Fh:]).to(h.dtype).float()
+        acc += topk_w[:, j:j + 1].float() * torch.einsum("tdf,tf->td", w_down[e].float(), a)
+    out.copy_(acc)
+
+
+def add2(x, y1, y2=None):
+    """x += y1 (+ y2), summed in fp32."""
+    s = y1.float() if y2 is None else y1.float() + y2.float()
+    x += s
