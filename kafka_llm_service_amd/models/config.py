@@ -126,13 +126,62 @@ BUDURAX_PRESETS: dict[str, dict] = {
 }
 
 
-def _from_json(path: Path):
-    """A config.json names its model class: ``"architecture": "Budurax"`` (models/budurax.py), else HF Llama / Mixtral."""
-    c = json.loads(path.read_text())
-    if str(c.get("architecture", "")).lower() == "budurax":
-        from kafka_llm_service_amd.models.budurax import BuduraxConfig
+def _lisorax(width: int, heads: int, kv_heads: int, n_layers: int, vocab: int, ff: int, experts: int = 8,
+             top: int = 2) -> dict:
+    """A Lisorax config dict at transformer-like sizes: 128-dim heads; layers cycle attention, rglru, attention that
+    borrows the first attention layer's keys and values, mlstm; every layer with routed experts of ``ff`` rows."""
+    moe = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
+    layers = []
+    for i in range(n_layers):
+        kind = i % 4
+        if kind in (0, 2):
+            m = {"heads": heads, "kv_heads": kv_heads, "dim": 128, "vdim": 128, "conv": 4, "scale": 128 ** -0.5,
+                 "softcap": 50.0, "q_temp": {"coef": 0.25, "every": 4096}}
+            if kind == 2:
+                m["kv_from"] = i - 2
+            layers.append({"type": "attention", "mixer": m, "mlp": moe})
+        elif kind == 1:
+            layers.append({"type": "rglru", "mixer": {"width": width, "blocks": max(1, width // 256), "conv": 4},
+                           "mlp": moe})
+        else:
+            layers.append({"type": "mlstm", "mixer": {"heads": max(1, width // 256), "dim": 128, "vdim": 256,
+                                                      "gate_cap": 10.0}, "mlp": moe})
+    return {"architecture": "Lisorax", "vocab": vocab, "width": width, "layers": layers, "norm": {"eps": 1e-6},
+            "embedding": {"scale": 1.0}, "canon": {"taps": 4}}
 
-        return BuduraxConfig.from_dict(c, name=path.parent.name)
+
+LISORAX_PRESETS: dict[str, dict] = {
+    # widths, heads and vocabularies of the Llama presets above; 8 experts of ff / 4 rows, top 2 (random init)
+    "lisorax-small": _lisorax(1024, 16, 4, 4, 128256, 896),
+    "lisorax-tiny": _lisorax(512, 8, 2, 4, 32000, 256, experts=4),
+}
+
+
+def _budurax_config(c: dict, name: str):
+    from kafka_llm_service_amd.models.budurax import BuduraxConfig
+
+    return BuduraxConfig.from_dict(c, name=name)
+
+
+def _lisorax_config(c: dict, name: str):
+    from kafka_llm_service_amd.models.lisorax import LisoraxConfig
+
+    return LisoraxConfig.from_dict(c, name=name)
+
+
+# config.json "architecture" (lower case) -> config class of a model family that names itself there
+ARCH_CONFIGS = {"budurax": _budurax_config, "lisorax": _lisorax_config}
+# model families whose kernels are built for float32 as well as bfloat16 (EngineConfig.dtype)
+FP32_ARCHS = ("budurax", "lisorax")
+
+
+def _from_json(path: Path):
+    """A config.json names its model class: ``"architecture": "Budurax"`` (models/budurax.py), ``"Lisorax"``
+    (models/lisorax.py), else HF Llama / Mixtral."""
+    c = json.loads(path.read_text())
+    make = ARCH_CONFIGS.get(str(c.get("architecture", "")).lower())
+    if make is not None:
+        return make(c, path.parent.name)
     return ModelConfig.from_hf(path)
 
 
@@ -140,12 +189,12 @@ def get_config(name: str):
     if name in PRESETS:
         return PRESETS[name]
     if name in BUDURAX_PRESETS:
-        from kafka_llm_service_amd.models.budurax import BuduraxConfig
-
-        return BuduraxConfig.from_dict(BUDURAX_PRESETS[name], name=name)
+        return _budurax_config(BUDURAX_PRESETS[name], name)
+    if name in LISORAX_PRESETS:
+        return _lisorax_config(LISORAX_PRESETS[name], name)
     p = Path(name)
     if p.is_dir() and (p / "config.json").exists():
         return _from_json(p / "config.json")
     if p.suffix == ".json" and p.exists():
         return _from_json(p)
-    raise KeyError(f"unknown model {name!r}; presets: {sorted(PRESETS)}")
+    raise KeyError(f"unknown model {name!r}; presets: {sorted(PRESETS) + sorted(BUDURAX_PRESETS) + sorted(LISORAX_PRESETS)}")

@@ -273,16 +273,21 @@ def build_model(cfg: ModelConfig, device, tp: int = 1, tp_rank: int = 0, seed: i
                 max_positions: int | None = None, dp_attention: tuple[int, int] | None = None, dtype=None):
     """``dp_attention = (ep, ep_rank)``: whole attention on this rank, experts sharded over the EP group.
     The model class follows ``cfg.arch`` (MODEL_CLASSES)."""
-    if cfg.arch == "budurax":
-        from kafka_llm_service_amd.models import budurax as bx
+    if cfg.arch in ("budurax", "lisorax"):  # segment-planned hybrid families: own tensor names, bf16 or fp32
+        if cfg.arch == "budurax":
+            from kafka_llm_service_amd.models import budurax as fam
 
-        model = bx.BuduraxLM(cfg, device, dtype=dtype or torch.bfloat16, tp=tp, tp_rank=tp_rank,
-                             max_positions=max_positions)
+            cls = fam.BuduraxLM
+        else:
+            from kafka_llm_service_amd.models import lisorax as fam
+
+            cls = fam.LisoraxLM
+        model = cls(cfg, device, dtype=dtype or torch.bfloat16, tp=tp, tp_rank=tp_rank, max_positions=max_positions)
         if weights:
-            return bx.load_checkpoint(model, weights)
+            return fam.load_checkpoint(model, weights)
         # small models (and every test) draw on the CPU; large ones directly on the device
         big = cfg.num_params() > 2e8 and torch.device(device).type == "cuda"
-        return model.load_tensors(bx.random_tensors(cfg, seed, device=device if big else "cpu"))
+        return model.load_tensors(fam.random_tensors(cfg, seed, device=device if big else "cpu"))
     if dtype not in (None, torch.bfloat16):
         raise ValueError(f"{cfg.arch} models run in bfloat16 only")
     model = TransformerLM(cfg, device, tp=tp, tp_rank=tp_rank, max_positions=max_positions)
