@@ -103,7 +103,9 @@ def parse(argv=None):
     ap.add_argument("--arch-prefill", default="512,2048,8192", help="prompt lengths of the prefill measurements")
     ap.add_argument("--arch-decode", default="16x2048,64x2048,64x8192",
                     help="decode measurements as <sequences>x<context tokens>")
-    ap.add_argument("--arch-models", default="budurax,llama")
+    ap.add_argument("--arch-models", default="budurax,llama",
+                    help="model families to measure, of budurax, llama, lisorax (sigmoid attention, rglru, mlstm "
+                         "layers with 8 routed experts, 2 per token, of half the dense feed-forward each)")
     return ap.parse_args(argv)
 
 
@@ -114,8 +116,9 @@ def arch_compare(args) -> int:
     import torch
 
     from kafka_llm_service_amd.engine.engine import EngineConfig, LLMEngine
-    from kafka_llm_service_amd.models.config import ModelConfig, _budurax
+    from kafka_llm_service_amd.models.config import ModelConfig, _budurax, _lisorax
     from kafka_llm_service_amd.models.budurax import BuduraxConfig
+    from kafka_llm_service_amd.models.lisorax import LisoraxConfig
 
     dev = "cuda:0" if torch.cuda.is_available() else "cpu"
     w, L = args.arch_width, args.arch_layers
@@ -124,6 +127,8 @@ def arch_compare(args) -> int:
     decodes = [tuple(int(v) for v in x.split("x")) for x in args.arch_decode.split(",") if x]
     need = max([max(prefills, default=0)] + [b * (c + 64) for b, c in decodes]) + 64
     cfgs = {"budurax": BuduraxConfig.from_dict(_budurax(w, heads, L, vocab, ff), name=f"budurax-w{w}-l{L}"),
+            "lisorax": LisoraxConfig.from_dict(_lisorax(w, heads, max(1, heads // 4), L, vocab, ff // 2 // 256 * 256),
+                                               name=f"lisorax-w{w}-l{L}"),
             "llama": ModelConfig(name=f"llama-w{w}-l{L}", hidden_size=w, intermediate_size=ff, num_layers=L,
                                  num_heads=heads, num_kv_heads=max(1, heads // 4), vocab_size=vocab,
                                  max_position_embeddings=131072, bos_token_id=1, eos_token_ids=[2])}
